@@ -1,0 +1,15 @@
+"""Python loader of the MI355X block-scaled FP8 GEMM library (libfp8gemm.so).
+
+The directory name contains a hyphen, so the package is loaded by path: the repository's
+__graft_entry__.load_package() registers it as module ``fp8_quant_matmul_amd``.
+Everything numerical happens in the HIP library behind the C ABI declared in
+include/fp8_block_gemm.h; this module only declares the ctypes prototypes and offers
+pointer-level helpers for torch tensors.  There is no CPU fallback: a missing library or
+a failing call raises.
+"""
+from .capi import (  # noqa: F401
+    Fp8GemmError,
+    KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY,
+    abi_symbols, build, convert_f32_to_e4m3fn, error_string, force_config, gemm, gemm_scalar,
+    last_kernel, lib, lib_path, release, select, set_workspace, workspace_bytes,
+)

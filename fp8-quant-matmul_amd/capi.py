@@ -1,0 +1,143 @@
+"""ctypes binding of include/fp8_block_gemm.h.
+
+`gemm(a, b, a_scale, b_scale, c, m, n, k)` keeps the reference launcher's argument order
+(/root/reference/check.cu:113, mn_large.hip:11).  Arguments are torch CUDA tensors (or raw
+integer device pointers); only their data_ptr() crosses the boundary.
+"""
+import ctypes as C
+import os
+import re
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5)
+
+
+class Fp8GemmError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = code
+        super().__init__(f"{where}: {error_string(code)} (code {code})")
+
+
+def lib_path():
+    return os.path.join(_HERE, "libfp8gemm.so")
+
+
+def build(force=True):
+    """Compile the HIP library for gfx950 (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", _HERE, "-j8"] + (["-B"] if force else [])
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
+
+
+def abi_symbols():
+    """Function names declared in include/fp8_block_gemm.h."""
+    hdr = os.path.join(_HERE, "..", "include", "fp8_block_gemm.h")
+    text = open(hdr).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fp8_[a-z0-9_]+)\s*\(", text)))
+
+
+def lib():
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = lib_path()
+    if not os.path.exists(path):
+        raise FileNotFoundError(
+            f"{path} is missing: build it with __graft_entry__.build() or `make -C {_HERE}`")
+    L = C.CDLL(path)
+    vp, fp, i, sz = C.c_void_p, C.c_void_p, C.c_int, C.c_size_t
+    L.fp8_block_gemm.restype = i
+    L.fp8_block_gemm.argtypes = [vp, vp, fp, fp, vp, i, i, i]
+    L.fp8_block_gemm_stream.restype = i
+    L.fp8_block_gemm_stream.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
+    L.fp8_block_gemm_scalar.restype = i
+    L.fp8_block_gemm_scalar.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
+    L.fp8_block_gemm_select.restype = i
+    L.fp8_block_gemm_select.argtypes = [i]
+    L.fp8_block_gemm_force_config.restype = i
+    L.fp8_block_gemm_force_config.argtypes = [i, i]
+    L.fp8_block_gemm_last_kernel.restype = C.c_char_p
+    L.fp8_block_gemm_last_kernel.argtypes = []
+    L.fp8_block_gemm_workspace_bytes.restype = sz
+    L.fp8_block_gemm_workspace_bytes.argtypes = [i, i, i]
+    L.fp8_block_gemm_set_workspace.restype = i
+    L.fp8_block_gemm_set_workspace.argtypes = [vp, sz]
+    L.fp8_block_gemm_release.restype = i
+    L.fp8_block_gemm_release.argtypes = []
+    L.fp8_convert_f32_to_e4m3fn.restype = i
+    L.fp8_convert_f32_to_e4m3fn.argtypes = [vp, vp, sz, vp]
+    L.fp8_block_gemm_error_string.restype = C.c_char_p
+    L.fp8_block_gemm_error_string.argtypes = [i]
+    L.fp8_block_gemm_abi_version.restype = i
+    L.fp8_block_gemm_abi_version.argtypes = []
+    L.fp8_gemm_host.restype = i
+    L.fp8_gemm_host.argtypes = [vp, vp, vp, vp, vp, sz, sz, sz, i]
+    _LIB = L
+    return L
+
+
+def error_string(code):
+    return lib().fp8_block_gemm_error_string(int(code)).decode()
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()
+
+
+def _check(rc, where):
+    if rc != 0:
+        raise Fp8GemmError(rc, where)
+
+
+def gemm(a, b, a_scale, b_scale, c, m, n, k, stream=None):
+    """C[m,n] bf16 = block-scaled A.B^T.  `stream` is a raw hipStream_t (int) or None for the
+    null stream."""
+    L = lib()
+    if stream is None:
+        rc = L.fp8_block_gemm(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k)
+    else:
+        rc = L.fp8_block_gemm_stream(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k,
+                                     stream)
+    _check(rc, "fp8_block_gemm")
+
+
+def gemm_scalar(a, b, a_scale, b_scale, c, m, n, k, stream=None):
+    rc = lib().fp8_block_gemm_scalar(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k,
+                                     stream)
+    _check(rc, "fp8_block_gemm_scalar")
+
+
+def select(kernel_id):
+    _check(lib().fp8_block_gemm_select(kernel_id), "fp8_block_gemm_select")
+
+
+def force_config(tile_variant=-1, ksplit=0):
+    _check(lib().fp8_block_gemm_force_config(tile_variant, ksplit), "fp8_block_gemm_force_config")
+
+
+def last_kernel():
+    return lib().fp8_block_gemm_last_kernel().decode()
+
+
+def workspace_bytes(m, n, k):
+    return int(lib().fp8_block_gemm_workspace_bytes(m, n, k))
+
+
+def set_workspace(ptr, nbytes):
+    _check(lib().fp8_block_gemm_set_workspace(_ptr(ptr), nbytes), "fp8_block_gemm_set_workspace")
+
+
+def release():
+    _check(lib().fp8_block_gemm_release(), "fp8_block_gemm_release")
+
+
+def convert_f32_to_e4m3fn(src, dst, count, stream=None):
+    _check(lib().fp8_convert_f32_to_e4m3fn(_ptr(src), _ptr(dst), count, stream),
+           "fp8_convert_f32_to_e4m3fn")

@@ -1,0 +1,319 @@
+// C ABI of the library (include/fp8_block_gemm.h): argument validation, kernel dispatch,
+// split-K workspace.  The dispatcher is the run-time counterpart of the reference's
+// compile-time kernel choice (#include "mn_large.hip" / "mn_small.hip", check.cu:13, and the
+// OPTION macro, mn_large.hip:9) and of gemmGPU's grid arithmetic (check.cu:92-114).
+#include "../../include/fp8_block_gemm.h"
+#include "launchers.h"
+
+#include <atomic>
+#include <cstdlib>
+#include <mutex>
+
+using namespace fp8gemm;
+
+namespace {
+
+constexpr int NUM_CU = 256;
+
+std::atomic<int> g_selected{FP8GEMM_KERNEL_AUTO};
+std::atomic<int> g_force_variant{-1};
+std::atomic<int> g_force_ksplit{0};
+thread_local const char* t_last_kernel = "none";
+thread_local char t_name_buf[64];
+
+std::mutex g_ws_mutex;
+float* g_ws_own = nullptr;       // library-owned workspace
+size_t g_ws_own_bytes = 0;
+float* g_ws_user = nullptr;      // caller-supplied workspace
+size_t g_ws_user_bytes = 0;
+
+struct Plan {
+    int family;   // FP8GEMM_KERNEL_*
+    int variant;  // TileVariant for the tile families
+    int ksplit;
+};
+
+int validate(const void* a, const void* b, const float* as, const float* bs, const void* c, int m,
+             int n, int k)
+{
+    if (!a || !b || !as || !bs || !c)
+        return FP8GEMM_E_NULLPTR;
+    if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
+        return FP8GEMM_E_SHAPE;
+    const long long lim = 0x7FFFFFFFll;
+    if ((long long)m * k > lim || (long long)n * k > lim || (long long)m * n > lim)
+        return FP8GEMM_E_TOOLARGE;
+    return FP8GEMM_OK;
+}
+
+// Estimated run time of a tile plan in units of "one 128-K block of a 256x256 tile".
+double tile_cost(const GemmArgs& g, int variant, int ksplit)
+{
+    int bm, bn;
+    tile_variant_dims(variant, &bm, &bn);
+    const int tiles = ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
+    const int nkb = g.k / 128;
+    const int kbs = (nkb + ksplit - 1) / ksplit;
+    const double per_kb = (double)bm * bn / 65536.0 * (bm * bn >= 65536 ? 1.0 : 1.15) + 0.08;
+    const double per_item = kbs * per_kb + 1.5 + (double)bm * bn / 65536.0 * (ksplit > 1 ? 1.0 : 0.5);
+    const long items = (long)tiles * ksplit;
+    const long rounds = (items + NUM_CU - 1) / NUM_CU;
+    double cost = rounds * per_item;
+    if (ksplit > 1)  // partial write + reduce read at a few TB/s, plus a second launch
+        cost += 3.0 + (double)g.m * g.n * ksplit * 8.0 / 3.0e12 / 0.9e-6;
+    return cost;
+}
+
+Plan make_plan(const GemmArgs& g, int selected)
+{
+    Plan p{FP8GEMM_KERNEL_SCALAR, 0, 1};
+    if (selected == FP8GEMM_KERNEL_SCALAR)
+        return p;
+    if (selected == FP8GEMM_KERNEL_SKINNY || (selected == FP8GEMM_KERNEL_AUTO && skinny_supports(g) && g.m <= 64)) {
+        if (skinny_supports(g)) {
+            p.family = FP8GEMM_KERNEL_SKINNY;
+            p.ksplit = skinny_ksplit(g);
+            return p;
+        }
+        if (selected == FP8GEMM_KERNEL_SKINNY) {
+            p.family = -1;
+            return p;
+        }
+    }
+    if (!tile_supports(g)) {
+        if (selected != FP8GEMM_KERNEL_AUTO)
+            p.family = -1;
+        return p;  // scalar fallback for shapes without 16-byte row alignment
+    }
+    const int fv = g_force_variant.load(), fk = g_force_ksplit.load();
+    const int nkb = g.k / 128;
+    double best = 1e300;
+    for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
+        if (fv >= 0 && v != fv)
+            continue;
+        if (tile_variant_name(v)[4] == '?')
+            continue;
+        for (int ks = 1; ks <= 16 && ks <= nkb; ++ks) {
+            if (fk > 0 && ks != (fk < nkb ? fk : nkb))
+                continue;
+            if (selected == FP8GEMM_KERNEL_LARGE && ks != 1)
+                continue;
+            if (selected == FP8GEMM_KERNEL_SPLITK && ks == 1 && nkb > 1)
+                continue;
+            // every split must own at least one K block
+            const int kbs = (nkb + ks - 1) / ks;
+            if ((ks - 1) * kbs >= nkb)
+                continue;
+            const double cst = tile_cost(g, v, ks);
+            if (cst < best) {
+                best = cst;
+                p.family = ks > 1 ? FP8GEMM_KERNEL_SPLITK : FP8GEMM_KERNEL_LARGE;
+                p.variant = v;
+                p.ksplit = ks;
+            }
+        }
+    }
+    if (best == 1e300)
+        p.family = -1;
+    return p;
+}
+
+// fp32 partial buffer of at least `bytes`, or nullptr with *err set
+float* get_workspace(size_t bytes, int* err)
+{
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    *err = FP8GEMM_OK;
+    if (g_ws_user) {
+        if (g_ws_user_bytes < bytes) {
+            *err = FP8GEMM_E_WORKSPACE;
+            return nullptr;
+        }
+        return g_ws_user;
+    }
+    if (g_ws_own_bytes < bytes) {
+        if (g_ws_own) {
+            // kernels of earlier calls may still read the old buffer
+            hipError_t e = hipDeviceSynchronize();
+            if (e != hipSuccess) {
+                *err = (int)e;
+                return nullptr;
+            }
+            (void)hipFree(g_ws_own);
+            g_ws_own = nullptr;
+            g_ws_own_bytes = 0;
+        }
+        void* p = nullptr;
+        hipError_t e = hipMalloc(&p, bytes);
+        if (e != hipSuccess) {
+            *err = (int)e;
+            return nullptr;
+        }
+        g_ws_own = static_cast<float*>(p);
+        g_ws_own_bytes = bytes;
+    }
+    return g_ws_own;
+}
+
+size_t plan_workspace_bytes(const GemmArgs& g, const Plan& p)
+{
+    if (p.ksplit <= 1)
+        return 0;
+    return (size_t)p.ksplit * g.m * g.n * sizeof(float);
+}
+
+int run(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k,
+        hipStream_t stream, int selected)
+{
+    int v = validate(a, b, as, bs, c, m, n, k);
+    if (v != FP8GEMM_OK)
+        return v;
+    GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), as, bs,
+               static_cast<uint16_t*>(c), m, n, k};
+    Plan p = make_plan(g, selected);
+    if (p.family < 0)
+        return FP8GEMM_E_KERNEL;
+    hipError_t e = hipSuccess;
+    switch (p.family) {
+    case FP8GEMM_KERNEL_SCALAR:
+        e = launch_scalar(g, stream);
+        t_last_kernel = "scalar";
+        break;
+    case FP8GEMM_KERNEL_SKINNY: {
+        float* ws = nullptr;
+        if (p.ksplit > 1) {
+            int err;
+            ws = get_workspace(plan_workspace_bytes(g, p), &err);
+            if (!ws)
+                return err;
+        }
+        e = launch_skinny(g, ws, stream);
+        t_last_kernel = "skinny";
+        break;
+    }
+    default: {
+        float* ws = nullptr;
+        if (p.ksplit > 1) {
+            int err;
+            ws = get_workspace(plan_workspace_bytes(g, p), &err);
+            if (!ws)
+                return err;
+        }
+        e = launch_tile(g, p.variant, p.ksplit, ws, stream);
+        if (e == hipSuccess && p.ksplit > 1)
+            e = launch_splitk_reduce(g, p.ksplit, ws, stream);
+        snprintf(t_name_buf, sizeof(t_name_buf), "%s_k%d", tile_variant_name(p.variant), p.ksplit);
+        t_last_kernel = t_name_buf;
+        break;
+    }
+    }
+    return (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fp8_block_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
+                   int m, int n, int k)
+{
+    return run(a, b, a_scale, b_scale, c, m, n, k, nullptr, g_selected.load());
+}
+
+int fp8_block_gemm_stream(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                          void* c, int m, int n, int k, void* stream)
+{
+    return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream),
+               g_selected.load());
+}
+
+int fp8_block_gemm_scalar(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                          void* c, int m, int n, int k, void* stream)
+{
+    return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream),
+               FP8GEMM_KERNEL_SCALAR);
+}
+
+int fp8_block_gemm_select(int kernel_id)
+{
+    if (kernel_id < FP8GEMM_KERNEL_AUTO || kernel_id > FP8GEMM_KERNEL_SKINNY)
+        return FP8GEMM_E_KERNEL;
+    g_selected.store(kernel_id);
+    return FP8GEMM_OK;
+}
+
+int fp8_block_gemm_force_config(int tile_variant, int ksplit)
+{
+    if (tile_variant >= TILE_VARIANT_COUNT || ksplit < 0 || ksplit > 64)
+        return FP8GEMM_E_KERNEL;
+    g_force_variant.store(tile_variant < 0 ? -1 : tile_variant);
+    g_force_ksplit.store(ksplit);
+    return FP8GEMM_OK;
+}
+
+const char* fp8_block_gemm_last_kernel(void) { return t_last_kernel; }
+
+size_t fp8_block_gemm_workspace_bytes(int m, int n, int k)
+{
+    if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
+        return 0;
+    // upper bound over every plan the dispatcher can pick: at most 16 K splits (64 when
+    // forced), each an m x n fp32 partial
+    int ks = g_force_ksplit.load() > 16 ? g_force_ksplit.load() : 16;
+    if (ks > k / 128)
+        ks = k / 128;
+    return (size_t)ks * m * n * sizeof(float);
+}
+
+int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)
+{
+    if (device_ptr && (reinterpret_cast<uintptr_t>(device_ptr) % 256) != 0)
+        return FP8GEMM_E_WORKSPACE;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    g_ws_user = static_cast<float*>(device_ptr);
+    g_ws_user_bytes = device_ptr ? bytes : 0;
+    return FP8GEMM_OK;
+}
+
+int fp8_block_gemm_release(void)
+{
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (g_ws_own) {
+        hipError_t e = hipDeviceSynchronize();
+        if (e != hipSuccess)
+            return (int)e;
+        e = hipFree(g_ws_own);
+        g_ws_own = nullptr;
+        g_ws_own_bytes = 0;
+        return (int)e;
+    }
+    return FP8GEMM_OK;
+}
+
+int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* stream)
+{
+    if (count == 0)
+        return FP8GEMM_OK;
+    if (!in || !out)
+        return FP8GEMM_E_NULLPTR;
+    return (int)launch_convert(in, static_cast<uint8_t*>(out), count, static_cast<hipStream_t>(stream));
+}
+
+const char* fp8_block_gemm_error_string(int code)
+{
+    switch (code) {
+    case FP8GEMM_OK: return "success";
+    case FP8GEMM_E_NULLPTR: return "a required pointer is NULL";
+    case FP8GEMM_E_SHAPE: return "m, n, k must be positive and k a multiple of 128";
+    case FP8GEMM_E_KERNEL: return "unknown kernel id or kernel not applicable to this shape";
+    case FP8GEMM_E_WORKSPACE: return "workspace too small or misaligned";
+    case FP8GEMM_E_TOOLARGE: return "operand exceeds 2^31-1 elements";
+    default: break;
+    }
+    if (code > 0)
+        return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown error code";
+}
+
+int fp8_block_gemm_abi_version(void) { return 1; }
+
+}  // extern "C"

@@ -1,0 +1,44 @@
+// The definition kernel: one thread per C element, sequential fp32 sum over each 128-wide
+// K block, scales applied per block, bf16 store.  Counterpart of ref_kernel
+// (/root/reference/check.cu:30-49); threads are mapped with n fastest so that the b reads
+// and the c stores of a wavefront are contiguous (the reference maps m fastest).
+#include "device_common.h"
+#include "launchers.h"
+
+namespace fp8gemm {
+
+__global__ void __launch_bounds__(256) scalar_gemm_kernel(const uint8_t* __restrict__ a,
+                                                          const uint8_t* __restrict__ b,
+                                                          const float* __restrict__ as,
+                                                          const float* __restrict__ bs,
+                                                          uint16_t* __restrict__ c, int m, int n, int k)
+{
+    int col = blockIdx.x * 64 + (threadIdx.x & 63);
+    int row = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (row >= m || col >= n)
+        return;
+    int sn = (n + KBLOCK - 1) / KBLOCK;
+    float result = 0.0f;
+    for (int k0 = 0; k0 < k; k0 += KBLOCK) {
+        float block = 0.0f;
+        for (int ii = 0; ii < KBLOCK; ++ii) {
+            float av = e4m3fn_to_f32(a[(size_t)row + (size_t)(k0 + ii) * m]);
+            float bv = e4m3fn_to_f32(b[(size_t)col + (size_t)(k0 + ii) * n]);
+            block = fmaf(av, bv, block);  // the product is exact in fp32, so fma == mul + add
+        }
+        float scaled = __fmul_rn(block, as[row + (size_t)(k0 / KBLOCK) * m]);
+        scaled = __fmul_rn(scaled, bs[col / KBLOCK + (size_t)(k0 / KBLOCK) * sn]);
+        result = __fadd_rn(result, scaled);
+    }
+    c[(size_t)row * n + col] = f32_to_bf16_bits(result);
+}
+
+hipError_t launch_scalar(const GemmArgs& g, hipStream_t s)
+{
+    dim3 grid((g.n + 63) / 64, (g.m + 3) / 4);
+    hipLaunchKernelGGL(scalar_gemm_kernel, grid, dim3(256), 0, s, g.a, g.b, g.a_scale, g.b_scale,
+                       g.c, g.m, g.n, g.k);
+    return hipGetLastError();
+}
+
+}  // namespace fp8gemm

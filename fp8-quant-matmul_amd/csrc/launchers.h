@@ -1,0 +1,41 @@
+// Internal (C++) launch functions behind the C ABI in include/fp8_block_gemm.h.
+// Each returns a hipError_t; none synchronises.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace fp8gemm {
+
+struct GemmArgs {
+    const uint8_t* a;
+    const uint8_t* b;
+    const float* a_scale;
+    const float* b_scale;
+    uint16_t* c;
+    int m, n, k;
+};
+
+// one thread per C element (check.cu:30-49)
+hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);
+
+// MFMA tile kernel family.  `variant` picks the workgroup tile; ksplit > 1 writes fp32
+// partial sums to `partial` ([ksplit][m][n]) instead of c and must be followed by
+// launch_splitk_reduce.
+enum TileVariant { TILE_256x256 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_256x192 = 3,
+                   TILE_128x192 = 4, TILE_VARIANT_COUNT };
+bool tile_supports(const GemmArgs& g);
+const char* tile_variant_name(int variant);
+void tile_variant_dims(int variant, int* bm, int* bn);
+hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, hipStream_t s);
+hipError_t launch_splitk_reduce(const GemmArgs& g, int ksplit, const float* partial, hipStream_t s);
+
+// tiny-M streaming kernel (decode shapes)
+bool skinny_supports(const GemmArgs& g);
+int skinny_ksplit(const GemmArgs& g);
+hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s);
+
+// fp32 -> e4m3fn (check.cu:17-22)
+hipError_t launch_convert(const float* in, uint8_t* out, size_t count, hipStream_t s);
+
+}  // namespace fp8gemm

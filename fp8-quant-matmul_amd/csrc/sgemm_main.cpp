@@ -1,0 +1,75 @@
+// Timing driver: the procedure of /root/reference/sgemm.cu:89-127 (10 launches bracketed by
+// events, first one dropped, mean of the remaining 9 in microseconds), on the full grid
+// (the reference's timed cases launch half of it, sgemm.cu:106).  Inputs are resident on the
+// device before the timed region.  Usage: sgemm M N K [runs]
+#include "host_harness.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#define CHECK(x)                                                                     \
+    do {                                                                             \
+        hipError_t e_ = (x);                                                         \
+        if (e_ != hipSuccess) {                                                      \
+            std::fprintf(stderr, "%s failed: %s\n", #x, hipGetErrorString(e_));      \
+            return 2;                                                                \
+        }                                                                            \
+    } while (0)
+
+int main(int argc, char** argv)
+{
+    using namespace harness;
+    size_t M = argc > 1 ? std::strtoul(argv[1], nullptr, 10) : 8192;
+    size_t N = argc > 2 ? std::strtoul(argv[2], nullptr, 10) : 4608;
+    size_t K = argc > 3 ? std::strtoul(argv[3], nullptr, 10) : 7168;
+    int runs = argc > 4 ? std::atoi(argv[4]) : 10;
+    const size_t nkb = K / 128, sn = (N + 127) / 128;
+
+    // byte patterns straight from the seed-7 stream: any finite e4m3 code
+    const auto fa = genMat(M * K > (1u << 22) ? (1u << 22) : M * K);
+    std::vector<uint8_t> a8(M * K), b8(N * K);
+    for (size_t i = 0; i < a8.size(); ++i)
+        a8[i] = (uint8_t)((int)(fa[i % fa.size()] * 12.f) & 0x77);
+    for (size_t i = 0; i < b8.size(); ++i)
+        b8[i] = (uint8_t)((int)(fa[(i * 7 + 3) % fa.size()] * 12.f) & 0x77);
+    std::vector<float> as(nkb * M, 0.01f), bs(nkb * sn, 0.02f);
+
+    void *da, *db, *das, *dbs, *dc;
+    CHECK(hipMalloc(&da, a8.size()));
+    CHECK(hipMalloc(&db, b8.size()));
+    CHECK(hipMalloc(&das, as.size() * 4));
+    CHECK(hipMalloc(&dbs, bs.size() * 4));
+    CHECK(hipMalloc(&dc, M * N * 2));
+    CHECK(hipMemcpy(da, a8.data(), a8.size(), hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(db, b8.data(), b8.size(), hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(das, as.data(), as.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(dbs, bs.data(), bs.size() * 4, hipMemcpyHostToDevice));
+
+    hipStream_t stream;
+    CHECK(hipStreamCreate(&stream));
+    hipEvent_t start, stop;
+    CHECK(hipEventCreate(&start));
+    CHECK(hipEventCreate(&stop));
+    float total = 0.f;
+    for (int i = 0; i < runs; ++i) {
+        CHECK(hipEventRecord(start, stream));
+        int rc = fp8_block_gemm_stream(da, db, (const float*)das, (const float*)dbs, dc, (int)M, (int)N,
+                                       (int)K, stream);
+        if (rc != 0) {
+            std::fprintf(stderr, "fp8_block_gemm: %s\n", fp8_block_gemm_error_string(rc));
+            return 2;
+        }
+        CHECK(hipEventRecord(stop, stream));
+        CHECK(hipEventSynchronize(stop));
+        float ms = 0.f;
+        CHECK(hipEventElapsedTime(&ms, start, stop));
+        if (i > 0)
+            total += ms;
+        std::printf("Run %d: %g ms\n", i + 1, ms);
+    }
+    double us = 1000.0 * total / (runs - 1);
+    std::printf("kernel %s: average of last %d runs: %.2f us, %.1f TFLOP/s\n",
+                fp8_block_gemm_last_kernel(), runs - 1, us, 2.0 * M * N * K / us * 1e-6);
+    return 0;
+}

@@ -1,0 +1,113 @@
+/*
+ * C ABI of the MI355X (gfx950) block-scaled FP8 GEMM.
+ *
+ *   C[M,N] (bf16, row-major) = sum over 128-wide K blocks kb of
+ *        a_scale[kb][m] * b_scale[kb][n/128] * ( A[m, kb-block] . B[n, kb-block] )
+ *
+ * Every pointer is a DEVICE pointer owned by the caller; the library never frees caller
+ * memory and fully overwrites c (no beta).  Layouts are the reference's, unchanged
+ * (/root/reference/check.cu:42-48):
+ *   a        fp8 e4m3fn (OCP) bytes, element (m,k) at  m + k*M          (M x K column-major)
+ *   b        fp8 e4m3fn (OCP) bytes, element (n,k) at  n + k*N          (N x K column-major)
+ *   a_scale  fp32, (kb,m)  at  m  + kb*M                                ([K/128][M])
+ *   b_scale  fp32, (kb,nb) at  nb + kb*ceil(N/128)                      ([K/128][ceil(N/128)])
+ *   c        bf16 bits, element (m,n) at m*N + n
+ * Preconditions: m, n, k > 0, k % 128 == 0, non-null pointers.  Any m and n are accepted.
+ *
+ * Return value: 0 on success; a negative FP8GEMM_E_* code for argument errors, detected
+ * before any device call; a positive hipError_t value when the HIP runtime reports one.
+ * Nothing is thrown across this boundary.  Launches are asynchronous on the given stream;
+ * no entry point synchronises the device.
+ */
+#ifndef FP8_BLOCK_GEMM_H
+#define FP8_BLOCK_GEMM_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP8GEMM_OK 0
+#define FP8GEMM_E_NULLPTR (-1)   /* a required pointer is NULL */
+#define FP8GEMM_E_SHAPE (-2)     /* m, n or k <= 0, or k not a multiple of 128 */
+#define FP8GEMM_E_KERNEL (-3)    /* unknown kernel id, or the kernel cannot run this shape */
+#define FP8GEMM_E_WORKSPACE (-4) /* caller-provided workspace too small or misaligned */
+#define FP8GEMM_E_TOOLARGE (-5)  /* m*k, n*k or m*n does not fit the 32-bit offsets used */
+
+/* Kernel ids for fp8_block_gemm_select (the run-time counterpart of the reference's
+ * compile-time OPTION / #include swap, mn_large.hip:9, check.cu:13). */
+#define FP8GEMM_KERNEL_AUTO 0   /* shape-based dispatch (default) */
+#define FP8GEMM_KERNEL_SCALAR 1 /* one thread per C element: ref_kernel, check.cu:30-49 */
+#define FP8GEMM_KERNEL_LARGE 2  /* MFMA tile kernel for large M and N: mn_large.hip:11 */
+#define FP8GEMM_KERNEL_SPLITK 3 /* MFMA tile kernel with the K range split over workgroups:
+                                   mn_small.hip:10 (small M*N, large K) */
+#define FP8GEMM_KERNEL_SKINNY 4 /* tiny-M streaming kernel (decode shapes) */
+
+/* The GEMM on the null stream.  Replaces the reference launch
+ * in_smem_kernel<<<grid, block, 0, 0>>>(A, B, As, Bs, C, M, N, K)
+ * (/root/reference/check.cu:106-114, kernel mn_large.hip:11 / mn_small.hip:10):
+ * same argument order and meaning. */
+int fp8_block_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                   void* c, int m, int n, int k);
+
+/* Same, on a caller-supplied hipStream_t (passed as void* so that this header needs no HIP
+ * include).  The reference only ever uses stream 0 (check.cu:113). */
+int fp8_block_gemm_stream(const void* a, const void* b, const float* a_scale,
+                          const float* b_scale, void* c, int m, int n, int k, void* stream);
+
+/* The scalar definition kernel: one thread per C element, sequential fp32 block sums.
+ * Replaces ref_kernel<<<...>>> (/root/reference/check.cu:30-49, launch check.cu:88). */
+int fp8_block_gemm_scalar(const void* a, const void* b, const float* a_scale,
+                          const float* b_scale, void* c, int m, int n, int k, void* stream);
+
+/* Force one kernel family for later calls from this process (FP8GEMM_KERNEL_*), or return
+ * to automatic dispatch.  Replaces the OPTION macro (/root/reference/mn_large.hip:9) and the
+ * `option` argument of gemmGPU (/root/reference/check.cu:51-52, 86-116). */
+int fp8_block_gemm_select(int kernel_id);
+
+/* Pin the MFMA tile kernels to one workgroup tile (0 = 256x256, 1 = 256x128, 2 = 128x128,
+ * -1 = choose by cost model) and one K-split count (0 = choose).  Benchmarking and test
+ * aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
+ * (/root/reference/mn_large.hip:1-8). */
+int fp8_block_gemm_force_config(int tile_variant, int ksplit);
+
+/* Name of the kernel variant the last successful call on this thread launched
+ * (static storage, never NULL).  No counterpart in the reference: diagnostics. */
+const char* fp8_block_gemm_last_kernel(void);
+
+/* Split-K kernels keep fp32 partial tiles in device memory.  By default the library owns a
+ * lazily grown buffer (allocated on first need, kept until fp8_block_gemm_release).
+ * A caller that must not allocate can supply its own: `bytes` must be at least
+ * fp8_block_gemm_workspace_bytes(m, n, k) for every later call, 256-byte aligned.
+ * Passing NULL returns to the library-owned buffer.  The reference has no workspace
+ * (its kernels do not split K: mn_small.hip:28). */
+size_t fp8_block_gemm_workspace_bytes(int m, int n, int k);
+int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes);
+int fp8_block_gemm_release(void);
+
+/* fp32 -> fp8 e4m3fn, round to nearest even, saturating to +-448; count elements.
+ * Replaces convert_float_to_fp8<<<M*K/256, 256>>> (/root/reference/check.cu:17-22, 83-84);
+ * unlike that launch it also converts a tail that is not a multiple of 256. */
+int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* stream);
+
+/* Text for a return code of any function above (static storage). */
+const char* fp8_block_gemm_error_string(int code);
+
+/* ABI version of this header: bumped on any incompatible change. */
+int fp8_block_gemm_abi_version(void);
+
+/* ---- host-buffer convenience layer: the reference's host launcher ----
+ * Counterpart of gemmGPU (/root/reference/check.cu:51-130): takes HOST buffers with fp32
+ * values for a and b (already in the column-major layouts above), allocates device
+ * memory, uploads, converts fp32 -> fp8 on the device, runs the kernel selected by
+ * `option`, downloads c (bf16 bits) and frees.  option: 2 = scalar definition kernel,
+ * 0 = automatic dispatch, 1 = same as 0 (the reference's "reverse" grid has no meaning
+ * here), or 100 + FP8GEMM_KERNEL_* to force a family.  Synchronous. */
+int fp8_gemm_host(unsigned short* c, const float* a, const float* b, const float* a_scale,
+                  const float* b_scale, size_t m, size_t n, size_t k, int option);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP8_BLOCK_GEMM_H */
