@@ -11,5 +11,5 @@ from .capi import (  # noqa: F401
     Fp8GemmError,
     KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY,
     abi_symbols, build, convert_f32_to_e4m3fn, error_string, force_config, gemm, gemm_scalar,
-    last_kernel, lib, lib_path, release, select, set_workspace, workspace_bytes,
+    last_kernel, lib, lib_path, plan, release, select, set_workspace, workspace_bytes,
 )

@@ -59,6 +59,8 @@ def lib():
     L.fp8_block_gemm_select.argtypes = [i]
     L.fp8_block_gemm_force_config.restype = i
     L.fp8_block_gemm_force_config.argtypes = [i, i]
+    L.fp8_block_gemm_plan.restype = i
+    L.fp8_block_gemm_plan.argtypes = [i, i, i, C.c_char_p, sz]
     L.fp8_block_gemm_last_kernel.restype = C.c_char_p
     L.fp8_block_gemm_last_kernel.argtypes = []
     L.fp8_block_gemm_workspace_bytes.restype = sz
@@ -120,6 +122,13 @@ def select(kernel_id):
 
 def force_config(tile_variant=-1, ksplit=0):
     _check(lib().fp8_block_gemm_force_config(tile_variant, ksplit), "fp8_block_gemm_force_config")
+
+
+def plan(m, n, k):
+    """Name of the kernel plan the dispatcher picks for this shape (no device access)."""
+    buf = C.create_string_buffer(64)
+    _check(lib().fp8_block_gemm_plan(m, n, k, buf, 64), "fp8_block_gemm_plan")
+    return buf.value.decode()
 
 
 def last_kernel():

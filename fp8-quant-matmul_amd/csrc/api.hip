@@ -6,6 +6,7 @@
 #include "launchers.h"
 
 #include <atomic>
+#include <cstdio>
 #include <cstdlib>
 #include <mutex>
 
@@ -187,7 +188,8 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
                 return err;
         }
         e = launch_skinny(g, ws, stream);
-        t_last_kernel = "skinny";
+        snprintf(t_name_buf, sizeof(t_name_buf), "skinny_k%d", p.ksplit);
+        t_last_kernel = t_name_buf;
         break;
     }
     default: {
@@ -251,6 +253,27 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit)
 }
 
 const char* fp8_block_gemm_last_kernel(void) { return t_last_kernel; }
+
+int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap)
+{
+    if (!name || cap == 0)
+        return FP8GEMM_E_NULLPTR;
+    if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
+        return FP8GEMM_E_SHAPE;
+    // aligned dummy addresses: only their alignment is inspected
+    GemmArgs g{reinterpret_cast<const uint8_t*>(uintptr_t(4096)), reinterpret_cast<const uint8_t*>(uintptr_t(4096)),
+               nullptr, nullptr, reinterpret_cast<uint16_t*>(uintptr_t(4096)), m, n, k};
+    Plan p = make_plan(g, g_selected.load());
+    if (p.family < 0)
+        return FP8GEMM_E_KERNEL;
+    if (p.family == FP8GEMM_KERNEL_SCALAR)
+        snprintf(name, cap, "scalar");
+    else if (p.family == FP8GEMM_KERNEL_SKINNY)
+        snprintf(name, cap, "skinny_k%d", p.ksplit);
+    else
+        snprintf(name, cap, "%s_k%d", tile_variant_name(p.variant), p.ksplit);
+    return FP8GEMM_OK;
+}
 
 size_t fp8_block_gemm_workspace_bytes(int m, int n, int k)
 {

@@ -13,6 +13,9 @@ __global__ void __launch_bounds__(256) scalar_gemm_kernel(const uint8_t* __restr
                                                           const float* __restrict__ bs,
                                                           uint16_t* __restrict__ c, int m, int n, int k)
 {
+    // no fused multiply-add anywhere but the explicit fmaf below: "result += block * as * bs"
+    // keeps its three separately rounded operations, as in a CPU build of the same line
+#pragma clang fp contract(off)
     int col = blockIdx.x * 64 + (threadIdx.x & 63);
     int row = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (row >= m || col >= n)
@@ -26,9 +29,9 @@ __global__ void __launch_bounds__(256) scalar_gemm_kernel(const uint8_t* __restr
             float bv = e4m3fn_to_f32(b[(size_t)col + (size_t)(k0 + ii) * n]);
             block = fmaf(av, bv, block);  // the product is exact in fp32, so fma == mul + add
         }
-        float scaled = __fmul_rn(block, as[row + (size_t)(k0 / KBLOCK) * m]);
-        scaled = __fmul_rn(scaled, bs[col / KBLOCK + (size_t)(k0 / KBLOCK) * sn]);
-        result = __fadd_rn(result, scaled);
+        float scaled = block * as[row + (size_t)(k0 / KBLOCK) * m];
+        scaled = scaled * bs[col / KBLOCK + (size_t)(k0 / KBLOCK) * sn];
+        result = result + scaled;
     }
     c[(size_t)row * n + col] = f32_to_bf16_bits(result);
 }

@@ -72,6 +72,12 @@ int fp8_block_gemm_select(int kernel_id);
  * (/root/reference/mn_large.hip:1-8). */
 int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 
+/* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
+ * 16-byte aligned operands into name[0..cap), e.g. "tile256x256_k1", "skinny_k1", "scalar".
+ * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart
+ * in the reference (its choice is made by editing the source, README.md:55). */
+int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap);
+
 /* Name of the kernel variant the last successful call on this thread launched
  * (static storage, never NULL).  No counterpart in the reference: diagnostics. */
 const char* fp8_block_gemm_last_kernel(void);

@@ -1,0 +1,88 @@
+"""Host-side behaviour of the C ABI that needs no GPU: the library loads, exports every
+symbol include/fp8_block_gemm.h declares, validates arguments before any device call, and
+the dispatcher's shape logic.  No compute call is made here."""
+import ctypes as C
+import os
+
+import pytest
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    L = pkg.lib()
+    names = pkg.abi_symbols()
+    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and len(names) >= 14
+    for name in names:
+        assert hasattr(L, name), f"{name} declared in the header but not exported"
+    assert L.fp8_block_gemm_abi_version() == 1
+
+
+def test_argument_validation_happens_before_any_device_call(pkg):
+    L = pkg.lib()
+    p = 4096  # never dereferenced
+    assert L.fp8_block_gemm(None, p, p, p, p, 16, 16, 128) == -1
+    assert L.fp8_block_gemm(p, p, p, p, None, 16, 16, 128) == -1
+    assert L.fp8_block_gemm(p, p, p, p, p, 0, 16, 128) == -2
+    assert L.fp8_block_gemm(p, p, p, p, p, 16, -3, 128) == -2
+    assert L.fp8_block_gemm(p, p, p, p, p, 16, 16, 100) == -2
+    assert L.fp8_block_gemm(p, p, p, p, p, 16, 16, 0) == -2
+    assert L.fp8_block_gemm_stream(p, p, p, p, p, 70000, 16, 65536, None) == -5
+    assert L.fp8_block_gemm_scalar(p, None, p, p, p, 16, 16, 128, None) == -1
+    assert L.fp8_gemm_host(None, p, p, p, p, 16, 16, 128, 0) == -1
+    assert L.fp8_gemm_host(p, p, p, p, p, 16, 16, 130, 0) == -2
+    assert L.fp8_convert_f32_to_e4m3fn(None, p, 10, None) == -1
+    assert L.fp8_convert_f32_to_e4m3fn(None, None, 0, None) == 0
+
+
+def test_error_strings_and_exception(pkg):
+    assert "NULL" in pkg.error_string(-1)
+    assert "128" in pkg.error_string(-2)
+    assert pkg.error_string(0) == "success"
+    with pytest.raises(pkg.Fp8GemmError) as ei:
+        pkg.gemm(4096, 4096, 4096, 4096, 4096, 16, 16, 64)
+    assert ei.value.code == -2
+
+
+def test_select_and_force_config_validate(pkg):
+    L = pkg.lib()
+    assert L.fp8_block_gemm_select(99) == -3
+    assert L.fp8_block_gemm_select(-1) == -3
+    assert L.fp8_block_gemm_force_config(99, 0) == -3
+    assert L.fp8_block_gemm_force_config(0, 1000) == -3
+    for kid in (1, 2, 3, 4, 0):
+        assert L.fp8_block_gemm_select(kid) == 0
+    assert L.fp8_block_gemm_force_config(-1, 0) == 0
+
+
+def test_workspace_contract(pkg):
+    L = pkg.lib()
+    assert pkg.workspace_bytes(0, 8, 128) == 0
+    assert pkg.workspace_bytes(64, 64, 128) == 64 * 64 * 4          # one K block: no split beyond 1
+    assert pkg.workspace_bytes(1024, 512, 2048) == 16 * 1024 * 512 * 4
+    assert L.fp8_block_gemm_set_workspace(4096 + 8, 1 << 20) == -4   # misaligned
+    assert L.fp8_block_gemm_set_workspace(None, 0) == 0
+    assert L.fp8_block_gemm_release() == 0                           # nothing allocated yet
+
+
+def test_dispatcher_plans(pkg):
+    pkg.select(pkg.KERNEL_AUTO)
+    pkg.force_config(-1, 0)
+    assert pkg.plan(8192, 4608, 7168).startswith("tile")
+    assert pkg.plan(8192, 4608, 7168).endswith("_k1")
+    assert pkg.plan(32, 7168, 2048).startswith("skinny")
+    assert pkg.plan(33, 100, 128) == "scalar"            # rows not 16-byte aligned
+    ks = int(pkg.plan(2048, 576, 7168).split("_k")[1])
+    assert ks > 1                                          # few tiles, long K: split
+    pkg.select(pkg.KERNEL_SCALAR)
+    assert pkg.plan(8192, 4608, 7168) == "scalar"
+    pkg.select(pkg.KERNEL_SKINNY)
+    with pytest.raises(pkg.Fp8GemmError):
+        pkg.plan(8192, 4608, 7168)                         # skinny cannot run M = 8192
+    pkg.select(pkg.KERNEL_AUTO)
+    pkg.force_config(1, 4)
+    assert pkg.plan(1024, 512, 2048) == "tile256x128_k4"
+    pkg.force_config(-1, 0)
+
+
+def test_header_cites_reference_for_every_entry_point(pkg):
+    hdr = open(os.path.join(os.path.dirname(pkg.lib_path()), "..", "include", "fp8_block_gemm.h")).read()
+    assert hdr.count("/root/reference/") >= 8

@@ -1,0 +1,273 @@
+"""GPU parity tests: every kernel family, through the C ABI, against the CPU oracle.
+
+Bars: the scalar definition kernel and the fp32->fp8 converter are bit-exact; the MFMA
+kernels satisfy max|C - ref| <= 1e-2 * max|ref| + 1e-3 (bf16 output rounding plus a
+different fp32 accumulation order inside a 128-wide block).
+"""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-3
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def _dev(*arrs):
+    import torch
+    return [torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in arrs]
+
+
+def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=False):
+    import torch
+    da, db, dsa, dsb = _dev(a, b, sa, sb)
+    dc = torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)  # NaN sentinel
+    _say(f"[gpu case] m={m} n={n} k={k} kernel={kernel} variant={variant} ksplit={ksplit} scalar={scalar}")
+    pkg.select(kernel)
+    pkg.force_config(variant, ksplit)
+    try:
+        if scalar:
+            pkg.gemm_scalar(da, db, dsa, dsb, dc, m, n, k)
+        else:
+            pkg.gemm(da, db, dsa, dsb, dc, m, n, k, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        name = pkg.last_kernel()
+    finally:
+        pkg.select(0)
+        pkg.force_config(-1, 0)
+    return dc.cpu().numpy().view(np.uint16), name
+
+
+def _assert_close(got, ref, what):
+    r = oracle.compare_bf16(got, ref, RTOL, ATOL)
+    assert r["bad"] == 0, (what, r)
+    return r
+
+
+# ------------------------------------------------------------------ scalar definition kernel
+@pytest.mark.parametrize("m,n,k", [(1, 1, 128), (48, 80, 128), (64, 128, 256), (33, 130, 384),
+                                   (128, 128, 256)])
+def test_scalar_kernel_is_bit_exact(pkg, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 100 + m)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, scalar=True)
+    assert name == "scalar"
+    assert np.array_equal(got, ref)
+
+
+def test_scalar_kernel_golden_fixture(pkg):
+    fx = np.load(os.path.join(os.path.dirname(__file__), "golden", "small_case.npz"))
+    m, n, k = [int(v) for v in fx["shape"]]
+    got, _ = _run(pkg, fx["a"], fx["b"], fx["a_scale"], fx["b_scale"], m, n, k, scalar=True)
+    assert np.array_equal(got, fx["c"])
+    got2, name = _run(pkg, fx["a"], fx["b"], fx["a_scale"], fx["b_scale"], m, n, k)
+    _assert_close(got2, fx["c"], name)
+
+
+# ------------------------------------------------------------------ MFMA tile kernels
+SHAPES = [(256, 256, 128), (256, 256, 256), (512, 768, 512), (272, 576, 384), (128, 128, 256),
+          (16, 16, 128), (1024, 192, 640), (304, 1040, 256), (64, 2048, 1024)]
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_tile_kernel(pkg, variant, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, m * 7 + n + variant, 1.0, 50.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant)
+    assert name.endswith("_k1"), name
+    _assert_close(got, ref, name)
+
+
+@pytest.mark.parametrize("variant,ksplit,m,n,k", [(2, 2, 256, 256, 512), (2, 4, 512, 512, 1024),
+                                                   (1, 3, 272, 576, 896), (0, 8, 256, 512, 2048),
+                                                   (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048)])
+def test_tile_kernel_split_k(pkg, variant, ksplit, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, m + n + k + ksplit)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SPLITK, variant=variant, ksplit=ksplit)
+    assert name.endswith(f"_k{ksplit}"), name
+    _assert_close(got, ref, name)
+
+
+@pytest.mark.parametrize("m,n,k", [(32, 7168, 2048), (16, 96, 512), (32, 576, 7168), (32, 32, 128),
+                                   (16, 1040, 384), (32, 4096, 256)])
+def test_skinny_kernel(pkg, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 900 + n)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY)
+    assert name.startswith("skinny")
+    _assert_close(got, ref, name)
+
+
+@pytest.mark.parametrize("m,n,k", [(33, 100, 128), (17, 129, 256), (100, 100, 384)])
+def test_unaligned_shapes_fall_back_to_the_scalar_kernel(pkg, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 5 + m)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k)
+    assert name == "scalar"
+    assert np.array_equal(got, ref)
+
+
+# ------------------------------------------------------------------ the five benchmark configurations
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+def test_benchmark_config_full_size(pkg, name):
+    m, n, k, a, b, sa, sb = oracle.make_config_inputs(name)
+    _say(f"[gpu case] {name}: oracle on {oracle.max_threads()} threads")
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, kname = _run(pkg, a, b, sa, sb, m, n, k)
+    r = _assert_close(got, ref, f"{name} {kname}")
+    _say(f"[gpu case] {name} {kname}: max_err={r['max_err']:.4g} bound={r['bound']:.4g}")
+    assert kname != "scalar"
+
+
+# ------------------------------------------------------------------ size-independent properties
+def test_results_are_bitwise_reproducible(pkg):
+    m, n, k = 512, 576, 2048
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 31)
+    for kw in (dict(kernel=2, variant=0), dict(kernel=3, variant=2, ksplit=4)):
+        x, _ = _run(pkg, a, b, sa, sb, m, n, k, **kw)
+        y, _ = _run(pkg, a, b, sa, sb, m, n, k, **kw)
+        assert np.array_equal(x, y)
+    a, b, sa, sb = oracle.make_inputs(32, 1024, 2048, 32)
+    x, _ = _run(pkg, a, b, sa, sb, 32, 1024, 2048, kernel=4)
+    y, _ = _run(pkg, a, b, sa, sb, 32, 1024, 2048, kernel=4)
+    assert np.array_equal(x, y)
+
+
+def test_n576_equals_zero_padded_n640_bit_for_bit(pkg):
+    m, k = 256, 1024
+    a, b, sa, sb = oracle.make_inputs(m, 576, k, 77)
+    bp = np.zeros((k, 640), np.uint8)
+    bp[:, :576] = b
+    x, _ = _run(pkg, a, b, sa, sb, m, 576, k, kernel=2, variant=2)
+    y, _ = _run(pkg, a, bp, sa, sb, m, 640, k, kernel=2, variant=2)
+    assert np.array_equal(x, y[:, :576])
+
+
+def test_power_of_two_scale_change_scales_the_result_exactly(pkg):
+    m, n, k = 256, 256, 512
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 88)
+    x, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=2, variant=0)
+    y, _ = _run(pkg, a, b, sa * 4, sb * 0.5, m, n, k, kernel=2, variant=0)
+    assert np.array_equal(oracle.bf16_decode(y), oracle.bf16_decode(x) * 2)
+
+
+def test_one_hot_inputs_pick_single_products(pkg):
+    m, n, k = 256, 384, 384
+    rng = np.random.RandomState(4)
+    sa = rng.uniform(1, 2, (3, m)).astype(np.float32)
+    sb = rng.uniform(1, 2, (3, 3)).astype(np.float32)
+    a = np.zeros((k, m), np.uint8)
+    b = np.zeros((k, n), np.uint8)
+    pts = [(0, 0, 0), (255, 383, 383), (17, 129, 130), (200, 256, 127)]
+    for (mi, ni, ki) in pts:
+        a[ki, mi] = 0x44  # 3.0... (code 0x44 = 1.5 * 2^1)
+        b[ki, ni] = 0x38  # 1.0
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    for kw in (dict(kernel=2, variant=0), dict(kernel=2, variant=2), dict(kernel=3, variant=1, ksplit=3)):
+        got, _ = _run(pkg, a, b, sa, sb, m, n, k, **kw)
+        assert np.array_equal(got, ref)
+    assert np.count_nonzero(ref) == len(pts)
+
+
+def test_nan_and_zero_scale_do_not_leak_into_other_elements(pkg):
+    m, n, k = 256, 256, 256
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 99)
+    a[5, 7] = 0x7F          # NaN in row 7
+    sa[1, 9] = 0.0          # K block 1 of row 9 contributes nothing
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=2, variant=0)
+    gf, rf = oracle.bf16_decode(got), oracle.bf16_decode(ref)
+    assert np.isnan(gf[7]).all() and np.isnan(rf[7]).all()
+    assert not np.isnan(np.delete(gf, 7, axis=0)).any()
+    _assert_close(np.delete(got, 7, axis=0), np.delete(ref, 7, axis=0), name)
+
+
+# ------------------------------------------------------------------ converter, host launcher, workspace, drivers
+def test_convert_kernel_is_bit_exact(pkg):
+    import torch
+    rng = np.random.RandomState(1)
+    codes = np.array([c for c in range(0x7F)], np.uint8)
+    vals = oracle.e4m3fn_decode(codes)
+    mids = ((vals[:-1].astype(np.float64) + vals[1:]) / 2).astype(np.float32)
+    x = np.concatenate([rng.standard_normal(100003).astype(np.float32) * 100, rng.standard_normal(5000).astype(np.float32) * 0.02,
+                        mids, -mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)),
+                        np.array([0.0, -0.0, 448, -448, 449, 464, 465, 1e30, -1e30, np.inf, -np.inf, 2.0 ** -10, 2.0 ** -11, 1e-30], np.float32)])
+    want = oracle.e4m3fn_encode(x)
+    dx = torch.from_numpy(x).cuda()
+    dq = torch.zeros(x.size, dtype=torch.uint8, device="cuda")
+    _say(f"[gpu case] convert {x.size} elements")
+    pkg.convert_f32_to_e4m3fn(dx, dq, x.size)
+    torch.cuda.synchronize()
+    assert np.array_equal(dq.cpu().numpy(), want)
+    xn = np.array([np.nan, 1.0, -np.nan], np.float32)
+    dxn = torch.from_numpy(xn).cuda()
+    dqn = torch.zeros(3, dtype=torch.uint8, device="cuda")
+    pkg.convert_f32_to_e4m3fn(dxn, dqn, 3)
+    q = dqn.cpu().numpy()
+    assert (q[0] & 0x7F) == 0x7F and q[1] == 0x38 and (q[2] & 0x7F) == 0x7F
+
+
+def test_host_launcher_matches_device_path(pkg):
+    """fp8_gemm_host (gemmGPU's counterpart): fp32 host values -> convert on device -> GEMM."""
+    m, n, k = 128, 128, 256
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 61)
+    af, bf = oracle.e4m3fn_decode(a), oracle.e4m3fn_decode(b)   # exactly representable
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    L = pkg.lib()
+    for option, exact in ((2, True), (0, False), (1, False), (102, False)):
+        c = np.zeros((m, n), np.uint16)
+        _say(f"[gpu case] fp8_gemm_host option={option}")
+        rc = L.fp8_gemm_host(c.ctypes.data, af.ctypes.data, bf.ctypes.data, sa.ctypes.data, sb.ctypes.data, m, n, k, option)
+        assert rc == 0
+        if exact:
+            assert np.array_equal(c, ref)
+        else:
+            _assert_close(c, ref, f"host option {option}")
+    assert L.fp8_gemm_host(c.ctypes.data, af.ctypes.data, bf.ctypes.data, sa.ctypes.data, sb.ctypes.data, m, n, k, 7) == -3
+
+
+def test_caller_workspace(pkg):
+    import torch
+    m, n, k = 256, 256, 1024
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 62)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    need = pkg.workspace_bytes(m, n, k)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    pkg.set_workspace(ws, need)
+    try:
+        got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=3, variant=2, ksplit=8)
+        _assert_close(got, ref, name)
+        pkg.set_workspace(ws, 1024)  # too small for an 8-way split
+        with pytest.raises(pkg.Fp8GemmError) as ei:
+            _run(pkg, a, b, sa, sb, m, n, k, kernel=3, variant=2, ksplit=8)
+        assert ei.value.code == -4
+    finally:
+        pkg.set_workspace(None, 0)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=3, variant=2, ksplit=8)
+    _assert_close(got, ref, name)
+    pkg.release()
+
+
+def test_check_driver_reproduces_the_reference_procedure(pkg):
+    """bin/check: seed-7 uniform(-5,5) inputs and scales, M=N=128, K=256, tolerance 100
+    (check.cu:137-177), plus a larger shape."""
+    exe = os.path.join(os.path.dirname(pkg.lib_path()), "bin", "check")
+    if not os.path.exists(exe):
+        pytest.skip("bin/check not built")
+    for args in ([], ["512", "384", "512", "100"]):
+        _say(f"[gpu case] bin/check {' '.join(args)}")
+        out = subprocess.run([exe] + args, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stdout + out.stderr
+        assert "2 matrices are equal" in out.stdout
