@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X block-scaled FP8 GEMM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4] [--no-shapes] [--no-cpu]
+
+A step is one GEMM call (C ABI, fp8_block_gemm_stream) on one configuration's synthetic
+inputs, already resident in HBM.  The headline workload is cfg4 (M=8192, N=4608, K=7168,
+the MFMA-utilisation shape); the other four configurations are timed too (shorter runs)
+and listed under "shapes" with the geomean latency.  One JSON line is printed.
+
+Timing: W untimed warm-up steps, then exactly K steps between two device synchronisations
+(wall clock -> ms_per_step, value) and between two HIP events recorded on the launch stream
+(-> roofline.achieved: algorithmic flops or bytes of one launch / average launch duration).
+cpu_baseline times the CPU oracle (the restatement of the reference's arithmetic) on a
+bounded row slice of the same workload with all host threads.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5033.0   # 256 CU x 2.4 GHz x 8192 flop/CU/clk (dense, v_mfma_f32_16x16x128_f8f6f4)
+PEAK_HBM_GBS = 8000.0
+HBM_BOUND = {"cfg5"}
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy
+# kernel of known size (profiles/): filled in per workload once measured, else null.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_work(m, n, k):
+    flops = 2.0 * m * n * k
+    sn = (n + 127) // 128
+    byts = m * k + n * k + 4 * (k // 128) * m + 4 * (k // 128) * sn + 2 * m * n
+    return flops, float(byts)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg4")
+    ap.add_argument("--no-shapes", action="store_true", help="time the headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus above 1 is not supported "
+              "(the GEMM shards by rows of A or 128-column blocks of B without exchange, "
+              "but no multi-GPU path is built)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import __graft_entry__ as ge
+    import oracle
+
+    pkg = ge.load_package()
+    pkg.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+    sptr = stream.cuda_stream
+
+    def prepare(name):
+        m, n, k, a, b, sa, sb = oracle.make_config_inputs(name)
+        dev = [torch.from_numpy(x).cuda() for x in (a, b, sa, sb)]
+        dc = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
+        return (m, n, k), (a, b, sa, sb), dev, dc
+
+    def step(dev, dc, shape):
+        pkg.gemm(dev[0], dev[1], dev[2], dev[3], dc, shape[0], shape[1], shape[2], sptr)
+
+    def parity(host, dc, shape, npts=8192):
+        m, n, k = shape
+        rs = np.random.RandomState(1234)
+        rows = rs.randint(0, m, npts).astype(np.int32)
+        cols = rs.randint(0, n, npts).astype(np.int32)
+        _, refh = oracle.ref_gemm_points(host[0], host[1], host[2], host[3], rows, cols, m, n, k)
+        got = dc.cpu().numpy().view(np.uint16)[rows, cols]
+        # bound from the sampled points' own max |ref|: stricter than the whole-matrix rule
+        r = oracle.compare_bf16(got, refh, 1e-2, 1e-3)
+        return {"points": npts, "max_err": r["max_err"], "bound": r["bound"], "pass": r["bad"] == 0}
+
+    def timed(dev, dc, shape, steps, warmup):
+        for _ in range(warmup):
+            step(dev, dc, shape)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(steps):
+            step(dev, dc, shape)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return wall_ms / steps, e0.elapsed_time(e1) / steps
+
+    def cold_latency_us(dev, dc, shape, reps=10):
+        """per-launch latency with caches flushed by a 1 GiB fill between launches"""
+        junk = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        ts = []
+        for i in range(reps):
+            junk.fill_(i)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            step(dev, dc, shape)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3)
+        del junk
+        ts.sort()
+        return ts[len(ts) // 2]
+
+    def shape_report(name, steps, warmup):
+        shape, host, dev, dc = prepare(name)
+        step(dev, dc, shape)
+        torch.cuda.synchronize()
+        par = parity(host, dc, shape)
+        wall_ms, ev_ms = timed(dev, dc, shape, steps, warmup)
+        flops, byts = algorithmic_work(*shape)
+        us = ev_ms * 1e3
+        rep = {
+            "name": name, "m": shape[0], "n": shape[1], "k": shape[2], "kernel": pkg.last_kernel(),
+            "latency_us": round(us, 2), "wall_us": round(wall_ms * 1e3, 2),
+            "tflops": round(flops / us * 1e-6, 1), "frac_fp8_peak": round(flops / us * 1e-6 / PEAK_FP8_TFLOPS, 4),
+            "gbs": round(byts / us * 1e-3, 1), "frac_hbm_peak": round(byts / us * 1e-3 / PEAK_HBM_GBS, 4),
+            "bound": "hbm" if name in HBM_BOUND else "mfma", "parity": par,
+        }
+        if name in HBM_BOUND:
+            cold = cold_latency_us(dev, dc, shape)
+            rep["cold_latency_us"] = round(cold, 2)
+            rep["cold_gbs"] = round(byts / cold * 1e-3, 1)
+        return rep, (shape, host, wall_ms, ev_ms)
+
+    main_rep, (shape, host, wall_ms, ev_ms) = shape_report(args.workload, args.steps, args.warmup)
+    m, n, k = shape
+    flops, byts = algorithmic_work(m, n, k)
+
+    shapes = [main_rep]
+    if not args.no_shapes:
+        for name in oracle.CONFIGS:
+            if name != args.workload:
+                rep, _ = shape_report(name, max(10, args.steps // 2), args.warmup)
+                shapes.append(rep)
+        shapes.sort(key=lambda r: r["name"])
+    geomean_us = math.exp(sum(math.log(r["latency_us"]) for r in shapes) / len(shapes))
+
+    hbm = args.workload in HBM_BOUND
+    if hbm:
+        achieved = byts / (ev_ms * 1e-3) * 1e-9
+        roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    else:
+        achieved = flops / (ev_ms * 1e-3) * 1e-12
+        roof = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4)}
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    roof["kernel"] = main_rep["kernel"]
+    roof["launch_us"] = round(ev_ms * 1e3, 2)
+    roof["algorithmic_flops"] = flops
+    roof["algorithmic_bytes"] = byts
+
+    cpu = None
+    if not args.no_cpu:
+        rows = min(m, 2048)
+        a, b, sa, sb = host
+        a_s = np.ascontiguousarray(a[:, :rows])
+        sa_s = np.ascontiguousarray(sa[:, :rows])
+        threads = oracle.max_threads()
+        t0 = time.perf_counter()
+        oracle.ref_gemm(a_s, b, sa_s, sb, rows, n, k, nthreads=threads)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(2.0 * rows * n * k / dt * 1e-12, 4), "unit": "TFLOP/s", "cores": threads,
+               "kind": "port", "seconds": round(dt, 3),
+               "sample": f"rows 0..{rows - 1} of A (of {m}), all {n} columns, K={k}: "
+                         f"{rows / m:.3f} of the workload's flops, CPU oracle oracle_ref_gemm"}
+
+    value = flops / (wall_ms * 1e-3) * 1e-12
+    out = {
+        "metric": "FP8 TFLOPS (block-scaled GEMM, dense) on the headline shape",
+        "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn x fp8_e4m3fn -> fp32 -> bf16",
+        "data": "synthetic (seeded N(0,1) -> bf16 -> 1x128 / 128x128 fp8 quantisation)",
+        "config": {"workload": f"{args.workload}: M={m} N={n} K={k}", "kernel": main_rep["kernel"],
+                   "frac_fp8_peak": round(value / PEAK_FP8_TFLOPS, 4)},
+        "parity": main_rep["parity"],
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "geomean_latency_us": round(geomean_us, 2),
+        "shapes": shapes,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
