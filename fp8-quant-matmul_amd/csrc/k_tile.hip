@@ -4,9 +4,9 @@
 // Data path (all of it differs from the reference, which scatters single bytes into LDS):
 //   * A ([K][M], m contiguous) and B ([K][N], n contiguous) tiles of 128 K-rows are copied
 //     global -> LDS with 16-byte buffer loads that write LDS directly (no VGPR round trip),
-//     keeping the global orientation: one LDS row per k, 256 bytes per row.  The 16-byte
-//     column chunk c of row r is stored at chunk position c ^ (2 * (r & 7)), which makes the
-//     transposing reads below bank-conflict free.
+//     keeping the global orientation: one LDS row per k, 128 or 256 bytes per row.  The
+//     16-byte column chunk c of row r is stored at chunk position c ^ swizzle(r), which makes
+//     the transposing reads below bank-conflict free (measured: 0 conflicts).
 //   * Operands are fetched with ds_read_b64_tr_b8: 16 lanes read an 8(k) x 16(m|n) byte
 //     patch and receive it transposed, i.e. lane i holds 8 consecutive k of column i.  Four
 //     such reads give the 32 bytes per lane that v_mfma_f32_32x32x64_f8f6f4 consumes.
@@ -15,42 +15,77 @@
 //   * Two MFMAs (K = 64 each) cover a 128-wide scale block of one 32x32 patch; the block sum
 //     lives in 16 registers for a moment and is folded into the running result with
 //     a_scale[kb][m] * b_scale[kb][n/128] by one FMA per element (mn_large.hip:100-106,
-//     mn_small.hip:85-88 do the same with a second full-size accumulator).  The 16-pass
-//     32x32x64 MFMA is used rather than the 8-pass 16x16x128 because a wave can issue about
-//     eight VALU instructions in the shadow of the former and none in that of the latter
-//     (measured), and this kernel needs ~11 VALU instructions per MFMA for the scale fold.
+//     mn_small.hip:85-88 do the same with a second full-size accumulator).
 //   * The MFMA computes the transposed patch (rows = n, columns = m) as mn_small.hip does,
 //     so that a lane owns one m (one a_scale value) and runs of 4 consecutive n (8-byte stores).
-//   * Two LDS stages: the copy of K block kb+1 is in flight while block kb is multiplied.
+//   * a_scale values of the tile travel through LDS with the stage (one extra 1 KiB copy), so
+//     the K loop holds no compiler-visible global load and every wait on the copies is the
+//     explicit one below.
+//   * NS LDS stages form a ring: the copies of K blocks kb+1 .. kb+NS-1 are in flight while
+//     block kb is multiplied.  Large tiles fit two stages; smaller tiles get three or four,
+//     which is what hides the global latency when a K block is only a few MFMAs long.
+//   * The copy instructions of a K block ride on the first MFMAs of an earlier block instead
+//     of being issued in one burst after the barrier (a burst queues up in the address unit
+//     and holds every wave back from its LDS reads).
 //
 // Work decomposition: grid.x = tiles (XCD-aware order), grid.y = K splits.
 #include "device_common.h"
 #include "launchers.h"
 
+#include <type_traits>
+
 namespace fp8gemm {
 
 namespace {
 
-constexpr int LDS_ROW = 256;                       // bytes per k-row of a stage (A or B)
-constexpr int LDS_MAT = KBLOCK * LDS_ROW;          // 32 KiB: one matrix, one stage
-constexpr int LDS_STAGE = 2 * LDS_MAT;             // A then B
-constexpr int LDS_TOTAL = 2 * LDS_STAGE;           // two stages, 128 KiB
 constexpr int NTHREADS = 512;
-constexpr int GROUP_M = 8;                         // tile rows per L2 locality group
+constexpr int GROUP_M = 8;  // tile rows per L2 locality group
 
-template <int BM, int BN, int WM, int WN, bool SPLIT>
+template <int BM, int BN, int WM, int WN, int NS>
+struct TileShape {
+    static constexpr int RSA = BM > 128 ? 256 : 128;  // LDS bytes per k-row of the A tile
+    static constexpr int RSB = BN > 128 ? 256 : 128;
+    static constexpr int MAT_A = KBLOCK * RSA;
+    static constexpr int MAT_B = KBLOCK * RSB;
+    static constexpr int SCALE_OFF = MAT_A + MAT_B;       // BM a_scale floats
+    static constexpr int STAGE = MAT_A + MAT_B + 1024;
+    static constexpr int LDS_BYTES = NS * STAGE;
+    static constexpr int NA = RSA / 64;                   // copy instructions per wave, A tile
+    static constexpr int NB = RSB / 64;
+    static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only)
+    static_assert(LDS_BYTES <= 160 * 1024, "stages exceed the 160 KiB of LDS");
+};
+
+// chunk swizzle of row r (0..7 within an 8-row group) for a row stride of RS bytes
+template <int RS>
+__device__ __forceinline__ int row_swizzle(int r)
+{
+    return RS == 256 ? 2 * (r & 7) : 2 * ((r >> 1) & 3);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
                  uint16_t* __restrict__ c, float* __restrict__ partial, int M, int N, int K,
                  int tiles_m, int tiles_n, int kb_per_split)
 {
+    using S = TileShape<BM, BN, WM, WN, NS>;
     static_assert(WM * WN == 8, "eight waves per workgroup");
+    static_assert(NS >= 2 && NS <= 4, "two to four LDS stages");
     constexpr int TM = BM / WM, TN = BN / WN;      // wave tile
     constexpr int MI = TM / 32, NJ = TN / 32;      // 32x32 patches per wave
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile is made of 32x32 patches");
     static_assert(TN <= 128, "a wave's n range touches at most two 128-wide scale blocks");
-    static_assert(BM <= 256 && BN <= 256, "LDS rows hold 256 bytes");
+    static_assert(BM <= 256 && BN <= 256, "LDS rows hold at most 256 bytes");
+    constexpr int RSA = S::RSA, RSB = S::RSB, NA = S::NA, NB = S::NB, NCOPY = S::NCOPY;
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     auto lds = LDS_PTR(uint8_t, smem);
@@ -79,39 +114,47 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     const int kb0 = blockIdx.y * kb_per_split;
     const int kb1 = (kb0 + kb_per_split < nkb) ? (kb0 + kb_per_split) : nkb;
 
-    // ---- global -> LDS copy plan.  A stage matrix is 32 slabs of 4 rows x 256 B; one
-    // 16-byte load per lane fills a slab (LDS address = slab base + lane*16).  Wave w owns
-    // slabs 4w..4w+3 of A and of B.  Lane l writes chunk position p = l & 15 of row r and
-    // therefore fetches column chunk p ^ (2 * (r & 7)).  Chunks outside the tile or the matrix get
-    // an out-of-range offset: the buffer load then returns zeros and touches no memory.
-    uint32_t voff_a[4], voff_b[4];
+    // ---- global -> LDS copy plan.  One 16-byte load per lane fills 1 KiB of LDS (LDS address
+    // = base + lane*16): 4 rows of 256 B or 8 rows of 128 B.  Wave w owns instructions
+    // NA*w .. NA*w+NA-1 of the A tile and likewise of B.  A lane writes chunk position p of
+    // row r and therefore fetches column chunk p ^ swizzle(r).  Chunks outside the tile or the
+    // matrix get an out-of-range offset: the buffer load then writes zeros and reads nothing.
+    uint32_t voff_a[NA], voff_b[NB];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int r = 16 * wave + 4 * q + (lane >> 4);
-        const int cc = (lane & 15) ^ (2 * (r & 7));
-        const bool va = (16 * cc < BM) && (m0 + 16 * cc < M);
-        const bool vb = (16 * cc < BN) && (n0 + 16 * cc < N);
-        voff_a[q] = va ? (uint32_t)(r * M + m0 + 16 * cc) : 0x80000000u;
-        voff_b[q] = vb ? (uint32_t)(r * N + n0 + 16 * cc) : 0x80000000u;
+    for (int q = 0; q < NA; ++q) {
+        const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
+        const int cc = (RSA == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSA>(r & 7);
+        const bool ok = (16 * cc < BM) && (m0 + 16 * cc < M);
+        voff_a[q] = ok ? (uint32_t)(r * M + m0 + 16 * cc) : 0x80000000u;
+    }
+#pragma unroll
+    for (int q = 0; q < NB; ++q) {
+        const int r = RSB == 256 ? (NB * wave + q) * 4 + (lane >> 4) : (NB * wave + q) * 8 + (lane >> 3);
+        const int cc = (RSB == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSB>(r & 7);
+        const bool ok = (16 * cc < BN) && (n0 + 16 * cc < N);
+        voff_b[q] = ok ? (uint32_t)(r * N + n0 + 16 * cc) : 0x80000000u;
     }
     const uint32_t a_bytes = (uint32_t)M * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
+    const uint32_t as_bytes = (uint32_t)nkb * (uint32_t)M * 4u;
+    const uint32_t voff_s =
+        (4 * lane < BM && m0 + 4 * lane < M) ? (uint32_t)((m0 + 4 * lane) * 4) : 0x80000000u;
 
-    // copy step q of K block kb into `stage`: q = 0..3 are the wave's A slabs, 4..7 its B slabs
-    auto issue_copy_step = [&](int stage, int kb, int q) {
-        const uint32_t dst = lds_base + (uint32_t)(stage * LDS_STAGE + wave * 4096);
-        if (q < 4) {
-            const uint32_t skip_a = (uint32_t)kb * KBLOCK * (uint32_t)M;
-            lds_dma16(make_rsrc_words(a + skip_a, a_bytes - skip_a), voff_a[q], dst + q * 1024);
-        } else {
-            const uint32_t skip_b = (uint32_t)kb * KBLOCK * (uint32_t)N;
-            lds_dma16(make_rsrc_words(b + skip_b, b_bytes - skip_b), voff_b[q - 4],
-                      dst + LDS_MAT + (q - 4) * 1024);
+    // copy instruction q (0..NCOPY-1) of K block kb into ring slot `slot`
+    auto copy_step = [&](int slot, int kb, int q) {
+        const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
+        if (q < NA) {
+            const uint32_t skip = (uint32_t)kb * KBLOCK * (uint32_t)M;
+            lds_dma16(make_rsrc_words(a + skip, a_bytes - skip), voff_a[q],
+                      stage + (uint32_t)((NA * wave + q) * 1024));
+        } else if (q < NA + NB) {
+            const uint32_t skip = (uint32_t)kb * KBLOCK * (uint32_t)N;
+            lds_dma16(make_rsrc_words(b + skip, b_bytes - skip), voff_b[q - NA],
+                      stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024));
+        } else if (wave == 0) {
+            const uint32_t skip = (uint32_t)kb * (uint32_t)M * 4u;
+            lds_dma16(make_rsrc_words(reinterpret_cast<const uint8_t*>(a_scale) + skip, as_bytes - skip),
+                      voff_s, stage + S::SCALE_OFF);
         }
-    };
-    auto issue_copy = [&](int stage, int kb) {
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            issue_copy_step(stage, kb, q);
     };
 
     // ---- transposing LDS reads.  Lane l = 16*g + i feeds MFMA row/column (l & 31) and k half
@@ -119,23 +162,24 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     // 64*ks + 32*(g>>1) + 8*t + (i>>1), 8-byte half (i & 1) of 16-byte chunk (patch chunk + (g&1)).
     // (row & 7) = (i >> 1) does not depend on t or ks: one address per patch plus immediates.
     const int g4 = lane >> 4, i16 = lane & 15;
-    const int swz = 2 * (i16 >> 1);
-    const uint32_t lane_off = (uint32_t)((32 * (g4 >> 1) + (i16 >> 1)) * LDS_ROW + (i16 & 1) * 8);
     uint32_t addr_a[MI], addr_b[NJ];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
-        addr_a[i] = lane_off + (uint32_t)((((wm * TM) / 16 + 2 * i + (g4 & 1)) ^ swz) * 16);
+        addr_a[i] = (uint32_t)((32 * (g4 >> 1) + (i16 >> 1)) * RSA + (i16 & 1) * 8 +
+                               ((((wm * TM) / 16 + 2 * i + (g4 & 1)) ^ row_swizzle<RSA>(i16 >> 1)) * 16));
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
-        addr_b[j] = LDS_MAT + lane_off + (uint32_t)((((wn * TN) / 16 + 2 * j + (g4 & 1)) ^ swz) * 16);
+        addr_b[j] = (uint32_t)(S::MAT_A + (32 * (g4 >> 1) + (i16 >> 1)) * RSB + (i16 & 1) * 8 +
+                               ((((wn * TN) / 16 + 2 * j + (g4 & 1)) ^ row_swizzle<RSB>(i16 >> 1)) * 16));
+    const uint32_t addr_s = S::SCALE_OFF + (uint32_t)((wm * TM + (lane & 31)) * 4);
 
-    // 32 bytes per lane of one operand for K step ks
-    auto read_frag = [&](uint32_t addr, int ks) -> v8i {
-        const uint32_t base = addr + (uint32_t)(ks * 64 * LDS_ROW);
+    // 32 bytes per lane of one operand for K step ks; rs = row stride of the matrix read
+    auto read_frag = [&](uint32_t addr, int ks, int rs) -> v8i {
+        const uint32_t base = addr + (uint32_t)(ks * 64 * rs);
         v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base));
-        v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 8 * LDS_ROW));
-        v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 16 * LDS_ROW));
-        v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 24 * LDS_ROW));
+        v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 8 * rs));
+        v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 16 * rs));
+        v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 24 * rs));
         return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
     };
 
@@ -152,16 +196,6 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
         patch_hi[j] = ((n_wave + 32 * j) >> 7) > (n_wave >> 7);
-    __amdgpu_buffer_rsrc_t ras = make_rsrc(a_scale, (uint32_t)nkb * (uint32_t)M * 4u);
-    // raw scale values of one K block; the a_scale * b_scale product is formed when used
-    auto load_scales = [&](int kb, float (&sa)[MI], float& sb_lo, float& sb_hi) {
-        sb_lo = b_scale[(size_t)kb * sn + nb_lo];
-        sb_hi = b_scale[(size_t)kb * sn + nb_hi];
-#pragma unroll
-        for (int i = 0; i < MI; ++i)
-            sa[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                                  ras, (uint32_t)((kb * M + m_lane + 32 * i) * 4), 0, 0));
-    };
 
     v16f acc[MI][NJ];
 #pragma unroll
@@ -173,72 +207,89 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                 acc[i][j][r] = 0.f;
     const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    // The copy and the scale loads of K block kb+1 are issued at the top of iteration kb and
-    // first needed at the top of iteration kb+1: a whole block of MFMA work hides them.
-    float sa_next[MI], sb_next = 0.f, sb_next_hi = 0.f;
+    // ---- prologue: the first NS-1 K blocks go into ring slots 0 .. NS-2
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
-        sa_next[i] = 0.f;
-    if (kb0 < kb1) {
-        issue_copy(0, kb0);
-        load_scales(kb0, sa_next, sb_next, sb_next_hi);
-    }
-
-    for (int kb = kb0; kb < kb1; ++kb) {
-        const int stage = (kb - kb0) & 1;
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's LDS copies have landed
-        __syncthreads();                     // everyone's have, and stage^1 is no longer read
-        float s[MI], s_hi[MI];
+    for (int p = 0; p < NS - 1; ++p)
+        if (kb0 + p < kb1) {
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            s[i] = sa_next[i] * sb_next;
-            s_hi[i] = sa_next[i] * sb_next_hi;
+            for (int q = 0; q < NCOPY; ++q)
+                copy_step(p, kb0 + p, q);
         }
-        const bool more = kb + 1 < kb1;
-        if (more)
-            load_scales(kb + 1, sa_next, sb_next, sb_next_hi);
 
-        // The eight copy instructions of the next K block are spread over the first half of
-        // this block's MFMAs: issued in one burst right after the barrier, the 64 copies of a
-        // workgroup queue up in the address unit and hold every wave back from its LDS reads.
-        constexpr int N_MFMA = MI * NJ * 2;
-        constexpr int SLOTS = (N_MFMA / 2 < 8) ? (N_MFMA / 2 < 1 ? 1 : N_MFMA / 2) : 8;
-        int slot = 0;
-        auto copy_slot = [&]() {
-            if (slot < SLOTS) {
-                if (more) {
+    int slot = 0;             // ring slot of block kb
+    int slot_fill = NS - 1;   // ring slot that block kb + NS - 1 goes into (= slot of kb - 1)
+
+    // One K block.  MORE = block kb+NS-1 exists and is copied here; two instantiations keep the
+    // steady-state body free of branches.
+    auto k_block = [&](auto more_tag, int kb) {
+        constexpr bool more = decltype(more_tag)::value;
+        // Block kb has landed once at most the copies of the younger blocks in flight are
+        // outstanding (loads complete in order).  NCOPY - 1 per block is exact for waves 1..7
+        // and one short for wave 0, which then waits for one more copy than it must.
+        if (more) {
+            wait_vmcnt<(NS - 2) * (NCOPY - 1)>();
+        } else {
+            const int younger = (kb1 - 1 - kb < NS - 2) ? (kb1 - 1 - kb) : (NS - 2);
+            if (NS >= 4 && younger >= 2)
+                wait_vmcnt<2 * (NCOPY - 1)>();
+            else if (NS >= 3 && younger >= 1)
+                wait_vmcnt<NCOPY - 1>();
+            else
+                wait_vmcnt<0>();
+        }
+        __syncthreads();  // everyone's copies of block kb landed; slot_fill is no longer read
+        const uint32_t so = (uint32_t)(slot * S::STAGE);
+        float sa[MI];
 #pragma unroll
-                    for (int q = 0; q < 8; ++q)
-                        if (q >= slot * 8 / SLOTS && q < (slot + 1) * 8 / SLOTS)
-                            issue_copy_step(stage ^ 1, kb + 1, q);
-                }
-                ++slot;
-            }
-        };
+        for (int i = 0; i < MI; ++i)
+            sa[i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
+        // wave-uniform addresses: scalar loads
+        const float sb_lo = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_lo)];
+        const float sb_hi = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_hi)];
 
-        const uint32_t so = (uint32_t)(stage * LDS_STAGE);
         v8i fa[MI][2];
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
-            fa[i][0] = read_frag(addr_a[i] + so, 0);
-            fa[i][1] = read_frag(addr_a[i] + so, 1);
+            fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
+            fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
         }
+        float s[MI], s_hi[MI];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            s[i] = sa[i] * sb_lo;
+            s_hi[i] = sa[i] * sb_hi;
+        }
+
+        // the wave's NCOPY copy instructions of block kb+NS-1 ride on the first MFMAs
+        constexpr int N_MFMA = MI * NJ * 2;
+        constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;  // copies behind each MFMA
+        int cq = 0;
+        auto copy_slot = [&](int n) {
+#pragma unroll
+            for (int u = 0; u < NCOPY; ++u)
+                if (u < n && cq < NCOPY) {
+                    if (more)
+                        copy_step(slot_fill, kb + NS - 1, cq);
+                    ++cq;
+                }
+        };
+
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            const v8i fb0 = read_frag(addr_b[j] + so, 0);
-            const v8i fb1 = read_frag(addr_b[j] + so, 1);
+            const v8i fb0 = read_frag(addr_b[j] + so, 0, RSB);
+            const v8i fb1 = read_frag(addr_b[j] + so, 1, RSB);
             v16f blk[MI];
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
                                                                           0, 0, 0);
-                copy_slot();
+                copy_slot(PER_MFMA);
             }
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
                                                                           0, 0, 0);
-                copy_slot();
+                copy_slot(PER_MFMA);
             }
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
@@ -248,7 +299,17 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                     acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
             }
         }
-    }
+        copy_slot(NCOPY);  // whatever is left (tiles with few MFMAs per K block)
+
+        slot_fill = slot;
+        slot = (slot + 1 == NS) ? 0 : slot + 1;
+    };
+    int kb = kb0;
+    for (; kb + NS - 1 < kb1; ++kb)
+        k_block(std::true_type{}, kb);
+    for (; kb < kb1; ++kb)
+        k_block(std::false_type{}, kb);
+
 
     // ---- epilogue: lane owns row m = .. + (lane & 31) and, per patch, four runs of 4 columns:
     // accumulator register 4*q + e is column 8*q + 4*(lane >> 5) + e of the patch
@@ -297,29 +358,30 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     *reinterpret_cast<uint2*>(c + i4) = pk;
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS>
 hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStream_t s)
 {
+    using S = TileShape<BM, BN, WM, WN, NS>;
     const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     const int nkb = g.k / KBLOCK;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     dim3 grid(tiles_m * tiles_n, ksplit);
     hipError_t e;
     if (ksplit > 1) {
-        auto kern = tile_gemm_kernel<BM, BN, WM, WN, true>;
+        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
         if (e != hipSuccess)
             return e;
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), S::LDS_BYTES, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
     } else {
-        auto kern = tile_gemm_kernel<BM, BN, WM, WN, false>;
+        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
         if (e != hipSuccess)
             return e;
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), S::LDS_BYTES, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
     }
     return hipGetLastError();
@@ -329,16 +391,16 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
 
 bool tile_supports(const GemmArgs& g)
 {
-    // 16-byte copies need every k-row of a and b to start 16-byte aligned
+    // 16-byte copies need every k-row of a, b and a_scale to start 16-byte aligned
     return g.m % 16 == 0 && g.n % 16 == 0 && (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.b) % 16 == 0) &&
+           (reinterpret_cast<uintptr_t>(g.a_scale) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
 }
 
 const char* tile_variant_name(int variant)
 {
     switch (variant) {
-    case TILE_256x256: return "tile256x256";
     case TILE_256x128: return "tile256x128";
     case TILE_128x128: return "tile128x128";
     case TILE_256x192: return "tile256x192";
@@ -350,7 +412,6 @@ const char* tile_variant_name(int variant)
 void tile_variant_dims(int variant, int* bm, int* bn)
 {
     switch (variant) {
-    case TILE_256x256: *bm = 256; *bn = 256; break;
     case TILE_256x128: *bm = 256; *bn = 128; break;
     case TILE_256x192: *bm = 256; *bn = 192; break;
     case TILE_128x192: *bm = 128; *bn = 192; break;
@@ -361,11 +422,10 @@ void tile_variant_dims(int variant, int* bm, int* bn)
 hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, hipStream_t s)
 {
     switch (variant) {
-    case TILE_256x256: return launch_variant<256, 256, 4, 2>(g, ksplit, partial, s);
-    case TILE_256x128: return launch_variant<256, 128, 4, 2>(g, ksplit, partial, s);
-    case TILE_128x128: return launch_variant<128, 128, 2, 4>(g, ksplit, partial, s);
-    case TILE_256x192: return launch_variant<256, 192, 4, 2>(g, ksplit, partial, s);
-    case TILE_128x192: return launch_variant<128, 192, 4, 2>(g, ksplit, partial, s);
+    case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, s);
+    case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, s);
+    case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, s);
+    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -1,7 +1,8 @@
 // Timing driver: the procedure of /root/reference/sgemm.cu:89-127 (10 launches bracketed by
 // events, first one dropped, mean of the remaining 9 in microseconds), on the full grid
 // (the reference's timed cases launch half of it, sgemm.cu:106).  Inputs are resident on the
-// device before the timed region.  Usage: sgemm M N K [runs]
+// device before the timed region.  Usage: sgemm M N K [runs [tile_variant [ksplit]]]
+// (tile_variant / ksplit pin the kernel plan as fp8_block_gemm_force_config does)
 #include "host_harness.h"
 
 #include <hip/hip_runtime.h>
@@ -24,6 +25,10 @@ int main(int argc, char** argv)
     size_t N = argc > 2 ? std::strtoul(argv[2], nullptr, 10) : 4608;
     size_t K = argc > 3 ? std::strtoul(argv[3], nullptr, 10) : 7168;
     int runs = argc > 4 ? std::atoi(argv[4]) : 10;
+    if (argc > 5 && fp8_block_gemm_force_config(std::atoi(argv[5]), argc > 6 ? std::atoi(argv[6]) : 0) != 0) {
+        std::fprintf(stderr, "bad tile_variant / ksplit\n");
+        return 2;
+    }
     const size_t nkb = K / 128, sn = (N + 127) / 128;
 
     // byte patterns straight from the seed-7 stream: any finite e4m3 code
