@@ -28,9 +28,14 @@ PEAK_FP8_TFLOPS = 5033.0   # 256 CU x 2.4 GHz x 8192 flop/CU/clk (dense, v_mfma_
 PEAK_HBM_GBS = 8000.0
 HBM_BOUND = {"cfg5"}
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy
-# kernel of known size (profiles/): filled in per workload once measured, else null.
-MEASURED_TRAFFIC_BYTES = {}
+# Bytes per launch that crossed the L2 <-> fabric boundary (Infinity Cache / HBM side), from
+# rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs (KiB per dispatch), each scaled by what the
+# same counter reads for a 1 GiB copy kernel: FETCH_SIZE reads 0.5 of the bytes copied
+# (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).  See profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg4": int((242049 * 2.0 + 75966 * 1.0) * 1024),   # 573 MB: 8 L2s refetch A/B panels
+    "cfg5": int((7462.75 * 2.0 + 448 * 1.0) * 1024),    # 15.7 MB: 1.04 x the algorithmic bytes
+}
 
 
 def algorithmic_work(m, n, k):
