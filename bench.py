@@ -2,11 +2,14 @@
 """Benchmark of the MI355X block-scaled FP8 GEMM.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4] [--no-shapes] [--no-cpu]
+                    [--no-challenge]
 
 A step is one GEMM call (C ABI, fp8_block_gemm_stream) on one configuration's synthetic
 inputs, already resident in HBM.  The headline workload is cfg4 (M=8192, N=4608, K=7168,
 the MFMA-utilisation shape); the other four configurations are timed too (shorter runs)
-and listed under "shapes" with the geomean latency.  One JSON line is printed.
+and listed under "shapes" with the geomean latency.  "challenge" holds the 18 shapes of the
+reference's own results table (/root/reference/README.md:15-25, measured there on an MI300X)
+with this library's latency on each and the geomean of the 18.  One JSON line is printed.
 
 Timing: W untimed warm-up steps, then exactly K steps between two device synchronisations
 (wall clock -> ms_per_step, value) and between two HIP events recorded on the launch stream
@@ -27,6 +30,14 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5033.0   # 256 CU x 2.4 GHz x 8192 flop/CU/clk (dense, v_mfma_f32_16x16x128_f8f6f4)
 PEAK_HBM_GBS = 8000.0
 HBM_BOUND = {"cfg5"}
+COLD_TOO = {"cfg1", "cfg3", "cfg5"}   # latency-bound shapes: also timed behind a cache flush
+
+# (k, n, MI300X latency in us for m=1024, for m=6144): the reference's published table,
+# /root/reference/README.md:15-25; its geomean over the 18 shapes is 136 us (README.md:13).
+CHALLENGE = [(7168, 1536, 147, 341), (1536, 3072, 50.6, 160), (7168, 576, 75.9, 173),
+             (256, 7168, 30.9, 88.6), (2048, 7168, 106, 426), (7168, 4608, 193, 948),
+             (2304, 7168, 120, 479), (7168, 512, 75.1, 163), (512, 4096, 30.9, 97.7)]
+CHALLENGE_REF_GEOMEAN_US = 136.0
 
 # Bytes per launch that crossed the L2 <-> fabric boundary (Infinity Cache / HBM side), from
 # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs (KiB per dispatch), each scaled by what the
@@ -36,6 +47,24 @@ MEASURED_TRAFFIC_BYTES = {
     "cfg4": int((242049 * 2.0 + 75966 * 1.0) * 1024),   # 573 MB: 8 L2s refetch A/B panels
     "cfg5": int((7462.75 * 2.0 + 448 * 1.0) * 1024),    # 15.7 MB: 1.04 x the algorithmic bytes
 }
+
+
+def max_sclk_mhz():
+    """highest "Max Clock Freq. (MHz)" rocminfo lists for a GPU agent, or None"""
+    import re
+    import subprocess
+    try:
+        text = subprocess.run(["/opt/rocm/bin/rocminfo"], capture_output=True, text=True, timeout=30).stdout
+    except Exception:
+        return None
+    best = None
+    for agent in text.split("*******")[1:]:
+        if "Device Type:             GPU" not in agent and not re.search(r"Device Type:\s+GPU", agent):
+            continue
+        mm = re.search(r"Max Clock Freq\. \(MHz\):\s+(\d+)", agent)
+        if mm:
+            best = max(best or 0, int(mm.group(1)))
+    return best
 
 
 def algorithmic_work(m, n, k):
@@ -53,6 +82,8 @@ def main():
     ap.add_argument("--workload", default="cfg4")
     ap.add_argument("--no-shapes", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-challenge", action="store_true",
+                    help="skip the 18 shapes of the reference's results table")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus above 1 is not supported "
@@ -74,7 +105,11 @@ def main():
     sptr = stream.cuda_stream
 
     def prepare(name):
-        m, n, k, a, b, sa, sb = oracle.make_config_inputs(name)
+        if isinstance(name, tuple):
+            m, n, k, seed = name
+            a, b, sa, sb = oracle.make_inputs(m, n, k, seed)
+        else:
+            m, n, k, a, b, sa, sb = oracle.make_config_inputs(name)
         dev = [torch.from_numpy(x).cuda() for x in (a, b, sa, sb)]
         dc = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
         return (m, n, k), (a, b, sa, sb), dev, dc
@@ -108,6 +143,18 @@ def main():
         wall_ms = (time.perf_counter() - t0) * 1e3
         return wall_ms / steps, e0.elapsed_time(e1) / steps
 
+    def launch_stats_us(dev, dc, shape, reps=20):
+        """median and minimum of single launches, each between its own pair of events"""
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(reps)]
+        for e0, e1 in ev:
+            e0.record(stream)
+            step(dev, dc, shape)
+            e1.record(stream)
+        torch.cuda.synchronize()
+        ts = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in ev)
+        return ts[len(ts) // 2], ts[0]
+
     def cold_latency_us(dev, dc, shape, reps=10):
         """per-launch latency with caches flushed by a 1 GiB fill between launches"""
         junk = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
@@ -140,11 +187,80 @@ def main():
             "gbs": round(byts / us * 1e-3, 1), "frac_hbm_peak": round(byts / us * 1e-3 / PEAK_HBM_GBS, 4),
             "bound": "hbm" if name in HBM_BOUND else "mfma", "parity": par,
         }
-        if name in HBM_BOUND:
+        med, mn = launch_stats_us(dev, dc, shape)
+        rep["single_launch_median_us"] = round(med, 2)
+        rep["single_launch_min_us"] = round(mn, 2)
+        if name in COLD_TOO:
             cold = cold_latency_us(dev, dc, shape)
             rep["cold_latency_us"] = round(cold, 2)
             rep["cold_gbs"] = round(byts / cold * 1e-3, 1)
         return rep, (shape, host, wall_ms, ev_ms)
+
+    def challenge_report(steps, warmup):
+        rows = []
+        for mi, m in enumerate((1024, 6144)):
+            for ci, (k, n, ref_1024, ref_6144) in enumerate(CHALLENGE):
+                shape, host, dev, dc = prepare((m, n, k, 2000 + 100 * mi + ci))
+                step(dev, dc, shape)
+                torch.cuda.synchronize()
+                par = parity(host, dc, shape, npts=2048)
+                _, ev_ms = timed(dev, dc, shape, steps, warmup)
+                us = ev_ms * 1e3
+                rows.append({"m": m, "n": n, "k": k, "kernel": pkg.last_kernel(),
+                             "latency_us": round(us, 2),
+                             "tflops": round(2.0 * m * n * k / us * 1e-6, 1),
+                             "reference_mi300x_us": ref_1024 if m == 1024 else ref_6144,
+                             "parity_pass": par["pass"]})
+                del dev, dc
+        geo = math.exp(sum(math.log(r["latency_us"]) for r in rows) / len(rows))
+        return {"shapes": rows, "geomean_latency_us": round(geo, 2),
+                "reference_mi300x_geomean_us": CHALLENGE_REF_GEOMEAN_US,
+                "note": "the reference's numbers are the author's MI300X measurements "
+                        "(context, different hardware)"}
+
+    def quantiser_report(steps, warmup):
+        """the device-side producers of the headline workload's operands (bf16 source)"""
+        out = []
+        for which, rows in (("a_1x128", m), ("b_128x128", n)):
+            x = torch.randn((rows, k), device="cuda", dtype=torch.float32).to(torch.bfloat16)
+            q = torch.empty((k, rows), dtype=torch.uint8, device="cuda")
+            ncol = rows if which == "a_1x128" else (rows + 127) // 128
+            sc = torch.empty((k // 128, ncol), dtype=torch.float32, device="cuda")
+            fn = pkg.quantize_a_1x128 if which == "a_1x128" else pkg.quantize_b_128x128
+            for _ in range(warmup):
+                fn(x, q, sc, rows, k, pkg.DTYPE_BF16, sptr)
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                fn(x, q, sc, rows, k, pkg.DTYPE_BF16, sptr)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / steps
+            nbytes = 3.0 * rows * k + 4.0 * sc.numel()
+            out.append({"kernel": "quantize_" + which, "rows": rows, "k": k, "source": "bf16",
+                        "latency_us": round(us, 2), "algorithmic_bytes": nbytes,
+                        "gbs": round(nbytes / us * 1e-3, 1),
+                        "frac_hbm_peak": round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4)})
+            del x, q, sc
+        return out
+
+    def launch_floor_us(reps=200):
+        """back-to-back launches of a one-workgroup kernel of this library"""
+        x = torch.zeros(256, dtype=torch.float32, device="cuda")
+        y = torch.zeros(256, dtype=torch.uint8, device="cuda")
+        for _ in range(10):
+            pkg.convert_f32_to_e4m3fn(x, y, 256, sptr)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            pkg.convert_f32_to_e4m3fn(x, y, 256, sptr)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
 
     main_rep, (shape, host, wall_ms, ev_ms) = shape_report(args.workload, args.steps, args.warmup)
     m, n, k = shape
@@ -158,6 +274,17 @@ def main():
                 shapes.append(rep)
         shapes.sort(key=lambda r: r["name"])
     geomean_us = math.exp(sum(math.log(r["latency_us"]) for r in shapes) / len(shapes))
+
+    challenge = None
+    if not args.no_challenge:
+        challenge = challenge_report(max(10, args.steps // 2), args.warmup)
+    floor_us = launch_floor_us()
+    quantisers = None if args.no_shapes else quantiser_report(max(10, args.steps // 2), args.warmup)
+    props = torch.cuda.get_device_properties(0)
+    device = {"name": props.name, "compute_units": props.multi_processor_count,
+              "max_sclk_mhz": max_sclk_mhz(),
+              "peak_fp8_tflops_assumed": PEAK_FP8_TFLOPS, "peak_hbm_gbs_assumed": PEAK_HBM_GBS,
+              "launch_floor_us": round(floor_us, 2)}
 
     hbm = args.workload in HBM_BOUND
     if hbm:
@@ -189,6 +316,14 @@ def main():
                "sample": f"rows 0..{rows - 1} of A (of {m}), all {n} columns, K={k}: "
                          f"{rows / m:.3f} of the workload's flops, CPU oracle oracle_ref_gemm"}
 
+        if not args.no_shapes:
+            m1, n1, k1, a1, b1, sa1, sb1 = oracle.make_config_inputs("cfg1")
+            t0 = time.perf_counter()
+            oracle.ref_gemm(a1, b1, sa1, sb1, m1, n1, k1, nthreads=1)
+            dt1 = time.perf_counter() - t0
+            cpu["single_thread_cfg1"] = {"seconds": round(dt1, 3),
+                                         "gflops": round(2.0 * m1 * n1 * k1 / dt1 * 1e-9, 2)}
+
     value = flops / (wall_ms * 1e-3) * 1e-12
     out = {
         "metric": "FP8 TFLOPS (block-scaled GEMM, dense) on the headline shape",
@@ -203,6 +338,9 @@ def main():
         "cpu_baseline": cpu,
         "geomean_latency_us": round(geomean_us, 2),
         "shapes": shapes,
+        "challenge": challenge,
+        "quantisers": quantisers,
+        "device": device,
     }
     print(json.dumps(out))
 

@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
 KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5)
+DTYPE_BF16, DTYPE_F32 = 0, 1
 
 
 class Fp8GemmError(RuntimeError):
@@ -71,6 +72,10 @@ def lib():
     L.fp8_block_gemm_release.argtypes = []
     L.fp8_convert_f32_to_e4m3fn.restype = i
     L.fp8_convert_f32_to_e4m3fn.argtypes = [vp, vp, sz, vp]
+    L.fp8_quantize_a_1x128.restype = i
+    L.fp8_quantize_a_1x128.argtypes = [vp, i, vp, fp, i, i, vp]
+    L.fp8_quantize_b_128x128.restype = i
+    L.fp8_quantize_b_128x128.argtypes = [vp, i, vp, fp, i, i, vp]
     L.fp8_block_gemm_error_string.restype = C.c_char_p
     L.fp8_block_gemm_error_string.argtypes = [i]
     L.fp8_block_gemm_abi_version.restype = i
@@ -150,3 +155,18 @@ def release():
 def convert_f32_to_e4m3fn(src, dst, count, stream=None):
     _check(lib().fp8_convert_f32_to_e4m3fn(_ptr(src), _ptr(dst), count, stream),
            "fp8_convert_f32_to_e4m3fn")
+
+
+def quantize_a_1x128(x, a, a_scale, m, k, dtype=DTYPE_BF16, stream=None):
+    """x [m][k] row-major (bf16 bits or fp32) -> a (fp8, element (m,k) at m + k*M) and
+    a_scale ([k/128][m]): to_float8_rowwise_scale of /root/reference/quantize.py:43-67 written
+    in the GEMM's layouts."""
+    _check(lib().fp8_quantize_a_1x128(_ptr(x), dtype, _ptr(a), _ptr(a_scale), m, k, stream),
+           "fp8_quantize_a_1x128")
+
+
+def quantize_b_128x128(x, b, b_scale, n, k, dtype=DTYPE_BF16, stream=None):
+    """x [n][k] row-major -> b (fp8 at n + k*N) and b_scale ([k/128][ceil(n/128)]):
+    to_float8_block_scale of /root/reference/quantize.py:16-41 written in the GEMM's layouts."""
+    _check(lib().fp8_quantize_b_128x128(_ptr(x), dtype, _ptr(b), _ptr(b_scale), n, k, stream),
+           "fp8_quantize_b_128x128")

@@ -1,0 +1,180 @@
+// Device-side quantisers: the producers of the GEMM's inputs.
+//
+//   1 x 128 groups along K per row   (to_float8_rowwise_scale, /root/reference/quantize.py:43-67)
+//   128 x 128 blocks                 (to_float8_block_scale,   /root/reference/quantize.py:16-41)
+//
+// Arithmetic of both, in fp32, with the OCP e4m3fn maximum 448:
+//   scale = 448 / max(amax, 1e-12);  q = fp8_rne(clamp(x * scale, -448, 448));  stored = 1 / scale
+//
+// The source x is row-major [rows][K] (K contiguous), bf16 or fp32.  The outputs are written
+// directly in the GEMM's layouts, which the reference produces with host-side transposes
+// (/root/reference/check.cu:164-167):  q at row + k*rows, the 1 x 128 scales at row + kb*rows,
+// the 128 x 128 scales at nb + kb*ceil(rows/128).
+//
+// One workgroup owns a 128-row x 128-k tile (one scale block, or 128 scale groups).  Sixteen
+// lanes read one row's 128 elements as 16- or 32-byte pieces (whole cache lines per row); the
+// fp8 bytes go through LDS transposed, and leave as 16-byte pieces of 128-byte row segments.
+// The kernel moves 2 (or 4) bytes in and 1 byte out per element: it is bound by HBM.
+#include "device_common.h"
+#include "launchers.h"
+
+namespace fp8gemm {
+
+namespace {
+
+constexpr int QTILE = 128;
+// LDS bytes per k-row of the transposed tile.  33 dwords: the byte stores of a wave (16 k-rows
+// 8 apart, 4 adjacent rows of the source) fall into 8 banks two deep, the dword reads into
+// distinct banks.
+constexpr int QSTRIDE = 132;
+
+__device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8])
+{
+    const uint4 w = *reinterpret_cast<const uint4*>(p);
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(u[i] << 16);
+        v[2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u);
+    }
+}
+
+__device__ __forceinline__ void load8(const float* p, float (&v)[8])
+{
+    const float4 lo = reinterpret_cast<const float4*>(p)[0];
+    const float4 hi = reinterpret_cast<const float4*>(p)[1];
+    v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+    v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+}
+
+__device__ __forceinline__ float clamp_pm448(float v)
+{
+    return fminf(fmaxf(v, -448.0f), 448.0f);
+}
+
+// BLOCK = false: one scale per row and tile (1 x 128).  BLOCK = true: one per tile (128 x 128).
+template <typename TIn, bool BLOCK>
+__global__ void __launch_bounds__(256)
+quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __restrict__ scale_out,
+                int rows, int K, int vec_store)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t tile[QTILE * QSTRIDE];
+    __shared__ float s_inv[QTILE];
+    __shared__ float s_red[4];
+
+    const int t = threadIdx.x;
+    const int c = t & 15;   // 8-element piece of the row's 128
+    const int r0 = t >> 4;  // row of the first pass; pass p handles row r0 + 16 p
+    const int row0 = blockIdx.x * QTILE;
+    const int kb = blockIdx.y;
+
+    float v[8][8];
+    float amax[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const int row = row0 + r0 + 16 * p;
+        if (row < rows) {
+            load8(x + (size_t)row * K + (size_t)kb * 128 + 8 * c, v[p]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                v[p][j] = 0.0f;
+        }
+        float a = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            a = fmaxf(a, __builtin_fabsf(v[p][j]));
+        amax[p] = a;
+    }
+
+    if (BLOCK) {
+        float a = amax[0];
+#pragma unroll
+        for (int p = 1; p < 8; ++p)
+            a = fmaxf(a, amax[p]);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1)
+            a = fmaxf(a, __shfl_xor(a, d));
+        if ((t & 63) == 0)
+            s_red[t >> 6] = a;
+        __syncthreads();
+        a = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+#pragma unroll
+        for (int p = 0; p < 8; ++p)
+            amax[p] = a;
+    } else {
+#pragma unroll
+        for (int p = 0; p < 8; ++p)
+#pragma unroll
+            for (int d = 1; d < 16; d <<= 1)
+                amax[p] = fmaxf(amax[p], __shfl_xor(amax[p], d));
+    }
+
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const int r = r0 + 16 * p;
+        const float scale = 448.0f / fmaxf(amax[p], 1e-12f);
+        int w0 = 0, w1 = 0;
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][0] * scale), clamp_pm448(v[p][1] * scale), w0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][2] * scale), clamp_pm448(v[p][3] * scale), w0, true);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][4] * scale), clamp_pm448(v[p][5] * scale), w1, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][6] * scale), clamp_pm448(v[p][7] * scale), w1, true);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            tile[(8 * c + j) * QSTRIDE + r] = (uint8_t)((uint32_t)w0 >> (8 * j));
+            tile[(8 * c + 4 + j) * QSTRIDE + r] = (uint8_t)((uint32_t)w1 >> (8 * j));
+        }
+        if (!BLOCK && c == 0)
+            s_inv[r] = 1.0f / scale;
+        if (BLOCK && t == 0 && p == 0)
+            scale_out[(size_t)kb * gridDim.x + blockIdx.x] = 1.0f / scale;
+    }
+    __syncthreads();
+
+    if (!BLOCK && t < QTILE && row0 + t < rows)
+        scale_out[(size_t)kb * rows + row0 + t] = s_inv[t];
+
+    // k-row kk of the tile: 128 bytes, one per source row; lane takes 16 of them
+    const int dq = t & 7;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int kk = (t >> 3) + 32 * pass;
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(tile + kk * QSTRIDE + 16 * dq);
+        const uint32_t w[4] = {src[0], src[1], src[2], src[3]};
+        const int first = row0 + 16 * dq;
+        const size_t o = (size_t)(kb * 128 + kk) * rows + first;
+        if (vec_store && first + 16 <= rows) {
+            *reinterpret_cast<uint4*>(q + o) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                if (first + j < rows)
+                    q[o + j] = (uint8_t)(w[j >> 2] >> (8 * (j & 3)));
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_quantize(const void* x, bool x_is_f32, uint8_t* q, float* scale_out, int rows,
+                           int k, bool block128, hipStream_t s)
+{
+    const dim3 grid((rows + QTILE - 1) / QTILE, k / 128);
+    const int vec_store = (rows % 16 == 0) && (reinterpret_cast<uintptr_t>(q) % 16 == 0);
+    if (x_is_f32) {
+        const float* xf = static_cast<const float*>(x);
+        if (block128)
+            hipLaunchKernelGGL((quantize_kernel<float, true>), grid, dim3(256), 0, s, xf, q, scale_out, rows, k, vec_store);
+        else
+            hipLaunchKernelGGL((quantize_kernel<float, false>), grid, dim3(256), 0, s, xf, q, scale_out, rows, k, vec_store);
+    } else {
+        const uint16_t* xh = static_cast<const uint16_t*>(x);
+        if (block128)
+            hipLaunchKernelGGL((quantize_kernel<uint16_t, true>), grid, dim3(256), 0, s, xh, q, scale_out, rows, k, vec_store);
+        else
+            hipLaunchKernelGGL((quantize_kernel<uint16_t, false>), grid, dim3(256), 0, s, xh, q, scale_out, rows, k, vec_store);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace fp8gemm

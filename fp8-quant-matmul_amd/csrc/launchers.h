@@ -38,4 +38,9 @@ hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s);
 // fp32 -> e4m3fn (check.cu:17-22)
 hipError_t launch_convert(const float* in, uint8_t* out, size_t count, hipStream_t s);
 
+// 1 x 128 (block128 = false) or 128 x 128 quantiser of a row-major [rows][k] matrix into the
+// GEMM's column-major fp8 layout and scale layout (quantize.py:16-67)
+hipError_t launch_quantize(const void* x, bool x_is_f32, uint8_t* q, float* scale_out, int rows,
+                           int k, bool block128, hipStream_t s);
+
 }  // namespace fp8gemm

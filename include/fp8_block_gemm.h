@@ -34,6 +34,12 @@ extern "C" {
 #define FP8GEMM_E_KERNEL (-3)    /* unknown kernel id, or the kernel cannot run this shape */
 #define FP8GEMM_E_WORKSPACE (-4) /* caller-provided workspace too small or misaligned */
 #define FP8GEMM_E_TOOLARGE (-5)  /* m*k, n*k or m*n does not fit the 32-bit offsets used */
+#define FP8GEMM_E_DTYPE (-6)     /* unknown FP8GEMM_DTYPE_* value */
+#define FP8GEMM_E_ALIGN (-7)     /* a source pointer is not 16-byte aligned */
+
+/* Element types of a quantiser's source matrix. */
+#define FP8GEMM_DTYPE_BF16 0
+#define FP8GEMM_DTYPE_F32 1
 
 /* Kernel ids for fp8_block_gemm_select (the run-time counterpart of the reference's
  * compile-time OPTION / #include swap, mn_large.hip:9, check.cu:13). */
@@ -96,6 +102,24 @@ int fp8_block_gemm_release(void);
  * Replaces convert_float_to_fp8<<<M*K/256, 256>>> (/root/reference/check.cu:17-22, 83-84);
  * unlike that launch it also converts a tail that is not a multiple of 256. */
 int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* stream);
+
+/* Quantise activations for the GEMM's `a` operand: x is [m][k] row-major (k contiguous),
+ * bf16 or fp32 (x_dtype = FP8GEMM_DTYPE_*), 16-byte aligned.  Per row and 128-wide K group:
+ * scale = 448 / max(amax, 1e-12), a = fp8_rne(clamp(x * scale, +-448)) written at m + k*M,
+ * a_scale = 1 / scale written at m + kb*M, all in fp32 arithmetic.  Replaces
+ * to_float8_rowwise_scale (/root/reference/quantize.py:43-67, with the e4m3fn maximum 448
+ * instead of fnuz's 240) together with the host-side transposes that bring its outputs into
+ * the kernel's layouts (row_to_col_major, /root/reference/check.cu:164-167). */
+int fp8_quantize_a_1x128(const void* x, int x_dtype, void* a, float* a_scale, int m, int k,
+                         void* stream);
+
+/* Quantise weights for the GEMM's `b` operand: x is [n][k] row-major, one scale per
+ * 128 x 128 block (a last block of fewer than 128 rows takes its amax over the rows that
+ * exist), b written at n + k*N, b_scale at nb + kb*ceil(N/128).  Replaces
+ * to_float8_block_scale (/root/reference/quantize.py:16-41; that function drops a partial
+ * last block, quantize.py:23-26) and the same transposes. */
+int fp8_quantize_b_128x128(const void* x, int x_dtype, void* b, float* b_scale, int n, int k,
+                           void* stream);
 
 /* Text for a return code of any function above (static storage). */
 const char* fp8_block_gemm_error_string(int code);

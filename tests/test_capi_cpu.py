@@ -10,10 +10,10 @@ import pytest
 def test_library_exports_every_declared_symbol(pkg):
     L = pkg.lib()
     names = pkg.abi_symbols()
-    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and len(names) >= 14
+    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and len(names) >= 16
     for name in names:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
-    assert L.fp8_block_gemm_abi_version() == 1
+    assert L.fp8_block_gemm_abi_version() == 2
 
 
 def test_argument_validation_happens_before_any_device_call(pkg):
@@ -31,6 +31,14 @@ def test_argument_validation_happens_before_any_device_call(pkg):
     assert L.fp8_gemm_host(p, p, p, p, p, 16, 16, 130, 0) == -2
     assert L.fp8_convert_f32_to_e4m3fn(None, p, 10, None) == -1
     assert L.fp8_convert_f32_to_e4m3fn(None, None, 0, None) == 0
+    for fn in (L.fp8_quantize_a_1x128, L.fp8_quantize_b_128x128):
+        assert fn(None, 0, p, p, 16, 128, None) == -1
+        assert fn(p, 0, p, None, 16, 128, None) == -1
+        assert fn(p, 0, p, p, 0, 128, None) == -2
+        assert fn(p, 0, p, p, 16, 192, None) == -2
+        assert fn(p, 0, p, p, 70000, 65536, None) == -5
+        assert fn(p, 7, p, p, 16, 128, None) == -6
+        assert fn(p + 2, 0, p, p, 16, 128, None) == -7
 
 
 def test_error_strings_and_exception(pkg):
