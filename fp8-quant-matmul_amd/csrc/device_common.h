@@ -64,9 +64,22 @@ __device__ __forceinline__ v4i make_rsrc_words(const void* base, uint32_t bytes)
 // it and would wait for the copy of the NEXT stage before reading the current one.  The
 // caller orders these copies itself (s_waitcnt vmcnt(0) + barrier before the data is read).
 // M0 is a reserved register that the compiler re-materialises before each of its own uses.
-__device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t voffset, uint32_t lds_addr)
+// soffset is a wave-uniform byte offset added to the global address only (not range checked,
+// not part of the LDS address).
+__device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t voffset, uint32_t lds_addr,
+                                          uint32_t soffset = 0)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %3 offen lds"
+                 :
+                 : "v"(voffset), "s"(rsrc), "s"(lds_addr), "s"(soffset)
+                 : "memory");
+}
+
+// The 4-byte-per-lane form: lane l's dword lands at lds_addr + 4*l.  Per-lane offsets are
+// free, so one instruction gathers 64 scattered dwords into a dense LDS table.
+__device__ __forceinline__ void lds_dma4(v4i rsrc, uint32_t voffset, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds"
                  :
                  : "v"(voffset), "s"(rsrc), "s"(lds_addr)
                  : "memory");

@@ -53,6 +53,9 @@ struct TileShape {
     static constexpr int NA = RSA / 64;                   // copy instructions per wave, A tile
     static constexpr int NB = RSB / 64;
     static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only)
+    // register-prefetch schedule only: b_scale pairs of the tile for up to 512 K blocks
+    static constexpr int BTAB_BLOCKS = 512;
+    static constexpr int BTAB_BYTES = (BTAB_BLOCKS + 32) * 8;
     static_assert(LDS_BYTES <= 160 * 1024, "stages exceed the 160 KiB of LDS");
 };
 
@@ -70,7 +73,7 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
+template <int BM, int BN, int WM, int WN, int NS, bool SPLIT, bool PF>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
@@ -139,21 +142,20 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     const uint32_t voff_s =
         (4 * lane < BM && m0 + 4 * lane < M) ? (uint32_t)((m0 + 4 * lane) * 4) : 0x80000000u;
 
-    // copy instruction q (0..NCOPY-1) of K block kb into ring slot `slot`
-    auto copy_step = [&](int slot, int kb, int q) {
+    // copy instruction q (0..NCOPY-1) of K block kb into ring slot `slot`.  The three buffer
+    // resources stay fixed; the K block's byte offset rides in the scalar offset operand.
+    const v4i rsrc_a = make_rsrc_words(a, a_bytes), rsrc_b = make_rsrc_words(b, b_bytes);
+    const v4i rsrc_s = make_rsrc_words(a_scale, as_bytes);
+    auto copy_step = [&](int slot, int kb, int q) __attribute__((always_inline)) {
         const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
         if (q < NA) {
-            const uint32_t skip = (uint32_t)kb * KBLOCK * (uint32_t)M;
-            lds_dma16(make_rsrc_words(a + skip, a_bytes - skip), voff_a[q],
-                      stage + (uint32_t)((NA * wave + q) * 1024));
+            lds_dma16(rsrc_a, voff_a[q], stage + (uint32_t)((NA * wave + q) * 1024),
+                      (uint32_t)kb * KBLOCK * (uint32_t)M);
         } else if (q < NA + NB) {
-            const uint32_t skip = (uint32_t)kb * KBLOCK * (uint32_t)N;
-            lds_dma16(make_rsrc_words(b + skip, b_bytes - skip), voff_b[q - NA],
-                      stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024));
+            lds_dma16(rsrc_b, voff_b[q - NA], stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
+                      (uint32_t)kb * KBLOCK * (uint32_t)N);
         } else if (wave == 0) {
-            const uint32_t skip = (uint32_t)kb * (uint32_t)M * 4u;
-            lds_dma16(make_rsrc_words(reinterpret_cast<const uint8_t*>(a_scale) + skip, as_bytes - skip),
-                      voff_s, stage + S::SCALE_OFF);
+            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)kb * (uint32_t)M * 4u);
         }
     };
 
@@ -174,7 +176,7 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     const uint32_t addr_s = S::SCALE_OFF + (uint32_t)((wm * TM + (lane & 31)) * 4);
 
     // 32 bytes per lane of one operand for K step ks; rs = row stride of the matrix read
-    auto read_frag = [&](uint32_t addr, int ks, int rs) -> v8i {
+    auto read_frag = [&](uint32_t addr, int ks, int rs) __attribute__((always_inline)) -> v8i {
         const uint32_t base = addr + (uint32_t)(ks * 64 * rs);
         v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base));
         v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 8 * rs));
@@ -207,132 +209,317 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                 acc[i][j][r] = 0.f;
     const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    // ---- prologue: the first NS-1 K blocks go into ring slots 0 .. NS-2
+    if constexpr (PF) {
+        // ---- register-prefetch schedule (small wave tiles: the K block is a handful of MFMAs,
+        // shorter than an LDS round trip, so the reads must not sit between barrier and MFMA).
+        // The fragments and scales of block kb+1 are read into a second register set while the
+        // MFMAs of block kb run on the first; the barrier at the top of a step therefore means
+        // "block kb+1 has landed and everyone has finished reading block kb", which frees the
+        // slot of block kb for block kb+NS: all NS slots hold blocks in flight.
+        const int nblk = kb1 - kb0;
+        const uint32_t btab = (uint32_t)(NS * S::STAGE);
+        {
+            // b_scale pairs (first, last 128-wide block the tile touches) of every K block:
+            // one gathering copy per 32 K blocks, entry j at btab + 8 j
+            const int nbt_lo = (n0 >> 7) < sn ? (n0 >> 7) : sn - 1;
+            const int nbt_hi = ((n0 + BN - 1) >> 7) < sn ? ((n0 + BN - 1) >> 7) : sn - 1;
+            const uint32_t bs_bytes = (uint32_t)nkb * (uint32_t)sn * 4u;
 #pragma unroll
-    for (int p = 0; p < NS - 1; ++p)
-        if (kb0 + p < kb1) {
-#pragma unroll
-            for (int q = 0; q < NCOPY; ++q)
-                copy_step(p, kb0 + p, q);
-        }
-
-    int slot = 0;             // ring slot of block kb
-    int slot_fill = NS - 1;   // ring slot that block kb + NS - 1 goes into (= slot of kb - 1)
-
-    // One K block.  MORE = block kb+NS-1 exists and is copied here; two instantiations keep the
-    // steady-state body free of branches.
-    auto k_block = [&](auto more_tag, int kb) {
-        constexpr bool more = decltype(more_tag)::value;
-        // Block kb has landed once at most the copies of the younger blocks in flight are
-        // outstanding (loads complete in order).  NCOPY - 1 per block is exact for waves 1..7
-        // and one short for wave 0, which then waits for one more copy than it must.
-        if (more) {
-            wait_vmcnt<(NS - 2) * (NCOPY - 1)>();
-        } else {
-            const int younger = (kb1 - 1 - kb < NS - 2) ? (kb1 - 1 - kb) : (NS - 2);
-            if (NS >= 4 && younger >= 2)
-                wait_vmcnt<2 * (NCOPY - 1)>();
-            else if (NS >= 3 && younger >= 1)
-                wait_vmcnt<NCOPY - 1>();
-            else
-                wait_vmcnt<0>();
-        }
-        __syncthreads();  // everyone's copies of block kb landed; slot_fill is no longer read
-        const uint32_t so = (uint32_t)(slot * S::STAGE);
-        float sa[MI];
-#pragma unroll
-        for (int i = 0; i < MI; ++i)
-            sa[i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
-        // wave-uniform addresses: scalar loads
-        const float sb_lo = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_lo)];
-        const float sb_hi = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_hi)];
-
-        v8i fa[MI][2];
-#pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
-            fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
-        }
-        float s[MI], s_hi[MI];
-#pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            s[i] = sa[i] * sb_lo;
-            s_hi[i] = sa[i] * sb_hi;
-        }
-
-        // the wave's NCOPY copy instructions of block kb+NS-1 ride on the first MFMAs
-        constexpr int N_MFMA = MI * NJ * 2;
-        constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;  // copies behind each MFMA
-        int cq = 0;
-        auto copy_slot = [&](int n) {
-#pragma unroll
-            for (int u = 0; u < NCOPY; ++u)
-                if (u < n && cq < NCOPY) {
-                    if (more)
-                        copy_step(slot_fill, kb + NS - 1, cq);
-                    ++cq;
+            for (int u = 0; u < S::BTAB_BLOCKS / 256; ++u) {
+                const int chunk = wave + 8 * u;
+                if (32 * chunk < nblk) {
+                    const int jb = 32 * chunk + (lane >> 1);
+                    const uint32_t vo =
+                        jb < nblk ? (uint32_t)(((kb0 + jb) * sn + ((lane & 1) ? nbt_hi : nbt_lo)) * 4)
+                                  : 0x80000000u;
+                    lds_dma4(make_rsrc_words(b_scale, bs_bytes), vo, lds_base + btab + (uint32_t)(chunk * 256));
                 }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < NS; ++p)
+            if (p < nblk) {
+#pragma unroll
+                for (int q = 0; q < NCOPY; ++q)
+                    copy_step(p, kb0 + p, q);
+            }
+        bool patch_hi_t[NJ];  // patch j lies in the tile's second b_scale block
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            patch_hi_t[j] = ((n_wave + 32 * j) >> 7) > (n0 >> 7);
+
+        v8i fa[2][MI][2], fb[2][NJ][2];
+        float sa[2][MI];
+        v2f sbp[2];
+        auto read_block = [&](auto set_tag, int slot_, int jlocal) __attribute__((always_inline)) {
+            constexpr int P = decltype(set_tag)::value;
+            const uint32_t so = (uint32_t)(slot_ * S::STAGE);
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                fa[P][i][0] = read_frag(addr_a[i] + so, 0, RSA);
+                fa[P][i][1] = read_frag(addr_a[i] + so, 1, RSA);
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                fb[P][j][0] = read_frag(addr_b[j] + so, 0, RSB);
+                fb[P][j][1] = read_frag(addr_b[j] + so, 1, RSB);
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+                sa[P][i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
+            sbp[P] = *LDS_PTR(v2f, lds + btab + (uint32_t)(8 * jlocal));
+        };
+        // wait until at most the copies of `y` younger blocks are outstanding
+        auto wait_younger = [&](int y) __attribute__((always_inline)) {
+            if (y <= 0)
+                wait_vmcnt<0>();
+            else if (y == 1)
+                wait_vmcnt<NCOPY - 1>();
+            else if (y == 2)
+                wait_vmcnt<2 * (NCOPY - 1)>();
+            else
+                wait_vmcnt<3 * (NCOPY - 1)>();
         };
 
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const v8i fb0 = read_frag(addr_b[j] + so, 0, RSB);
-            const v8i fb1 = read_frag(addr_b[j] + so, 1, RSB);
-            v16f blk[MI];
-#pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
-                                                                          0, 0, 0);
-                copy_slot(PER_MFMA);
+        wait_younger((nblk < NS ? nblk : NS) - 1);
+        __syncthreads();
+        read_block(std::integral_constant<int, 0>{}, 0, 0);
+        int slot = 0;
+
+        // One K block on register set P.  FILL: 1 = block kb+NS exists and is copied here,
+        // 0 = decided at run time (the last NS+1 blocks of the range).
+        auto step = [&](auto set_tag, auto fill_tag, int kb) __attribute__((always_inline)) {
+            constexpr int P = decltype(set_tag)::value;
+            constexpr bool steady = decltype(fill_tag)::value;
+            const bool fill = steady || (kb + NS < kb1);
+            if (steady) {
+                wait_vmcnt<(NS - 2) * (NCOPY - 1)>();  // blocks kb+2 .. kb+NS-1 may be in flight
+            } else if (kb + 1 < kb1) {
+                const int last = (kb + NS - 1 < kb1 - 1) ? (kb + NS - 1) : (kb1 - 1);
+                wait_younger(last - (kb + 1));
             }
+            __syncthreads();
+            const int slot_next = (slot + 1 == NS) ? 0 : slot + 1;
+            // past the last block this reads a stale slot into registers nobody uses
+            read_block(std::integral_constant<int, 1 - P>{}, slot_next, kb - kb0 + 1);
+
+            float s[MI], s_hi[MI];
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
-                blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
-                                                                          0, 0, 0);
-                copy_slot(PER_MFMA);
+                s[i] = sa[P][i] * sbp[P].x;
+                s_hi[i] = sa[P][i] * sbp[P].y;
             }
+            constexpr int N_MFMA = MI * NJ * 2;
+            constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;
+            int cq = 0;
+            auto copy_slot = [&](int n) __attribute__((always_inline)) {
 #pragma unroll
+                for (int u = 0; u < NCOPY; ++u)
+                    if (u < n && cq < NCOPY) {
+                        if (fill)
+                            copy_step(slot, kb + NS, cq);
+                        ++cq;
+                    }
+            };
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                v16f blk[MI];
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[P][j][0], fa[P][i][0], zero16,
+                                                                              0, 0, 0, 0, 0, 0);
+                    copy_slot(PER_MFMA);
+                }
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[P][j][1], fa[P][i][1], blk[i],
+                                                                              0, 0, 0, 0, 0, 0);
+                    copy_slot(PER_MFMA);
+                }
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    const float sc = patch_hi_t[j] ? s_hi[i] : s[i];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
+                }
+            }
+            copy_slot(NCOPY);
+            slot = slot_next;
+        };
+        using Set0 = std::integral_constant<int, 0>;
+        using Set1 = std::integral_constant<int, 1>;
+        int kb = kb0;
+        for (; kb + NS + 1 < kb1; kb += 2) {  // both blocks of the pair have a block NS ahead
+            step(Set0{}, std::true_type{}, kb);
+            step(Set1{}, std::true_type{}, kb + 1);
+        }
+        for (; kb < kb1; kb += 2) {
+            step(Set0{}, std::false_type{}, kb);
+            if (kb + 1 < kb1)
+                step(Set1{}, std::false_type{}, kb + 1);
+        }
+    } else {
+        // ---- prologue: the first NS-1 K blocks go into ring slots 0 .. NS-2
+    #pragma unroll
+        for (int p = 0; p < NS - 1; ++p)
+            if (kb0 + p < kb1) {
+    #pragma unroll
+                for (int q = 0; q < NCOPY; ++q)
+                    copy_step(p, kb0 + p, q);
+            }
+
+        int slot = 0;             // ring slot of block kb
+        int slot_fill = NS - 1;   // ring slot that block kb + NS - 1 goes into (= slot of kb - 1)
+
+        // One K block.  MORE = block kb+NS-1 exists and is copied here; two instantiations keep the
+        // steady-state body free of branches.
+        auto k_block = [&](auto more_tag, int kb) {
+            constexpr bool more = decltype(more_tag)::value;
+            // Block kb has landed once at most the copies of the younger blocks in flight are
+            // outstanding (loads complete in order).  NCOPY - 1 per block is exact for waves 1..7
+            // and one short for wave 0, which then waits for one more copy than it must.
+            if (more) {
+                wait_vmcnt<(NS - 2) * (NCOPY - 1)>();
+            } else {
+                const int younger = (kb1 - 1 - kb < NS - 2) ? (kb1 - 1 - kb) : (NS - 2);
+                if (NS >= 4 && younger >= 2)
+                    wait_vmcnt<2 * (NCOPY - 1)>();
+                else if (NS >= 3 && younger >= 1)
+                    wait_vmcnt<NCOPY - 1>();
+                else
+                    wait_vmcnt<0>();
+            }
+            __syncthreads();  // everyone's copies of block kb landed; slot_fill is no longer read
+            const uint32_t so = (uint32_t)(slot * S::STAGE);
+            float sa[MI];
+    #pragma unroll
+            for (int i = 0; i < MI; ++i)
+                sa[i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
+            // wave-uniform addresses: scalar loads
+            const float sb_lo = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_lo)];
+            const float sb_hi = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_hi)];
+
+            v8i fa[MI][2];
+    #pragma unroll
             for (int i = 0; i < MI; ++i) {
-                const float sc = patch_hi[j] ? s_hi[i] : s[i];
+                fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
+                fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
+            }
+            float s[MI], s_hi[MI];
+    #pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                s[i] = sa[i] * sb_lo;
+                s_hi[i] = sa[i] * sb_hi;
+            }
+
+            // the wave's NCOPY copy instructions of block kb+NS-1 ride on the first MFMAs
+            constexpr int N_MFMA = MI * NJ * 2;
+            constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;  // copies behind each MFMA
+            int cq = 0;
+            auto copy_slot = [&](int n) {
+    #pragma unroll
+                for (int u = 0; u < NCOPY; ++u)
+                    if (u < n && cq < NCOPY) {
+                        if (more)
+                            copy_step(slot_fill, kb + NS - 1, cq);
+                        ++cq;
+                    }
+            };
+
+    #pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const v8i fb0 = read_frag(addr_b[j] + so, 0, RSB);
+                const v8i fb1 = read_frag(addr_b[j] + so, 1, RSB);
+                v16f blk[MI];
+    #pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
+                                                                              0, 0, 0);
+                    copy_slot(PER_MFMA);
+                }
+    #pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
+                                                                              0, 0, 0);
+                    copy_slot(PER_MFMA);
+                }
+    #pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    const float sc = patch_hi[j] ? s_hi[i] : s[i];
+    #pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
+                }
+            }
+            copy_slot(NCOPY);  // whatever is left (tiles with few MFMAs per K block)
+
+            slot_fill = slot;
+            slot = (slot + 1 == NS) ? 0 : slot + 1;
+        };
+        int kb = kb0;
+        for (; kb + NS - 1 < kb1; ++kb)
+            k_block(std::true_type{}, kb);
+        for (; kb < kb1; ++kb)
+            k_block(std::false_type{}, kb);
+
+
+    }
+
+    // ---- epilogue.  A lane owns row m = .. + (lane & 31) and, per patch, four runs of 4 columns
+    // (accumulator register 4*q + e is column 8*q + 4*(lane >> 5) + e of the patch): stored
+    // straight from the registers that would be 8- or 16-byte pieces of 32 different rows per
+    // instruction.  The tile therefore goes through the (now idle) LDS ring, row-major with a
+    // padded row stride that keeps the writes conflict free, and leaves as 16 bytes per lane
+    // along whole rows of the tile.  A tile larger than the ring is written in two halves.
+    constexpr int ESZ = SPLIT ? 4 : 2;
+    constexpr int CROW = BN * ESZ + (SPLIT ? 16 : 8);  // LDS bytes per tile row
+    constexpr int HALVES = (BM * CROW <= S::LDS_BYTES) ? 1 : 2;
+    constexpr int HROWS = BM / HALVES;
+    static_assert(HROWS * CROW <= S::LDS_BYTES, "half a tile must fit the ring");
+    static_assert(HROWS % 32 == 0, "a 32-row patch lies in one half");
+    constexpr int CPR = BN * ESZ / 16;                 // 16-byte chunks per tile row
+    constexpr int CHUNKS = HROWS * CPR;
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
+    for (int h = 0; h < HALVES; ++h) {
+        __syncthreads();  // nobody reads the ring (or the previous half) any more
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const int prow = wm * TM + 32 * i;  // first tile row of the patch
+            if (prow / HROWS == h) {
+                const uint32_t rbase = (uint32_t)((prow - h * HROWS + (lane & 31)) * CROW);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int col = wn * TN + 32 * j + 8 * q + 4 * (lane >> 5);
+                        const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                       acc[i][j][4 * q + 3]};
+                        if (SPLIT) {
+                            *LDS_PTR(v4f, lds + rbase + col * 4) = v;
+                        } else {
+                            v2i pk = {(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3])};
+                            *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
+                        }
+                    }
             }
         }
-        copy_slot(NCOPY);  // whatever is left (tiles with few MFMAs per K block)
-
-        slot_fill = slot;
-        slot = (slot + 1 == NS) ? 0 : slot + 1;
-    };
-    int kb = kb0;
-    for (; kb + NS - 1 < kb1; ++kb)
-        k_block(std::true_type{}, kb);
-    for (; kb < kb1; ++kb)
-        k_block(std::false_type{}, kb);
-
-
-    // ---- epilogue: lane owns row m = .. + (lane & 31) and, per patch, four runs of 4 columns:
-    // accumulator register 4*q + e is column 8*q + 4*(lane >> 5) + e of the patch
+        __syncthreads();
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
-        const int mrow = m_lane + 32 * i;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int ncol = n0 + wn * TN + 32 * j + 8 * q + 4 * (lane >> 5);
-                if (mrow < M && ncol < N) {
-                    const size_t o = (size_t)mrow * N + ncol;
-                    const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                   acc[i][j][4 * q + 3]};
-                    if (SPLIT) {
-                        *reinterpret_cast<v4f*>(partial + (size_t)blockIdx.y * M * N + o) = v;
-                    } else {
-                        uint2 pk;
-                        pk.x = pack_bf16x2(v[0], v[1]);
-                        pk.y = pack_bf16x2(v[2], v[3]);
-                        *reinterpret_cast<uint2*>(c + o) = pk;
-                    }
+        for (int it = 0; it < (CHUNKS + NTHREADS - 1) / NTHREADS; ++it) {
+            const int idx = it * NTHREADS + (int)threadIdx.x;
+            const int row = idx / CPR, ch = idx - row * CPR;
+            const int mrow = m0 + h * HROWS + row;
+            const int ncol = n0 + ch * (16 / ESZ);
+            if (idx < CHUNKS && mrow < M && ncol < N) {
+                const size_t o = (size_t)mrow * N + ncol;
+                if (SPLIT) {
+                    const v4f v = *LDS_PTR(v4f, lds + row * CROW + ch * 16);
+                    *reinterpret_cast<v4f*>(partial + (size_t)blockIdx.y * M * N + o) = v;
+                } else {
+                    const v2i lo = *LDS_PTR(v2i, lds + row * CROW + ch * 16);
+                    const v2i hi = *LDS_PTR(v2i, lds + row * CROW + ch * 16 + 8);
+                    *reinterpret_cast<v4i*>(c + o) = (v4i){lo.x, lo.y, hi.x, hi.y};
                 }
             }
         }
@@ -358,30 +545,36 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     *reinterpret_cast<uint2*>(c + i4) = pk;
 }
 
-template <int BM, int BN, int WM, int WN, int NS>
+template <int BM, int BN, int WM, int WN, int NS, bool PF = false>
 hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStream_t s)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
+    constexpr int LDS_TOTAL = S::LDS_BYTES + (PF ? S::BTAB_BYTES : 0);
+    static_assert(LDS_TOTAL <= 160 * 1024, "stages and scale table exceed the 160 KiB of LDS");
     const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     const int nkb = g.k / KBLOCK;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
+    if constexpr (PF) {
+        if (kb_per_split > S::BTAB_BLOCKS)  // scale table too small: the plain schedule has no limit
+            return launch_variant<BM, BN, WM, WN, NS, false>(g, ksplit, partial, s);
+    }
     dim3 grid(tiles_m * tiles_n, ksplit);
     hipError_t e;
     if (ksplit > 1) {
-        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
+        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true, PF>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
         if (e != hipSuccess)
             return e;
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), S::LDS_BYTES, s, g.a, g.b, g.a_scale, g.b_scale,
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
     } else {
-        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
+        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false, PF>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
         if (e != hipSuccess)
             return e;
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), S::LDS_BYTES, s, g.a, g.b, g.a_scale, g.b_scale,
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
     }
     return hipGetLastError();
@@ -395,7 +588,7 @@ bool tile_supports(const GemmArgs& g)
     return g.m % 16 == 0 && g.n % 16 == 0 && (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.b) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.a_scale) % 16 == 0) &&
-           (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
+           (reinterpret_cast<uintptr_t>(g.c) % 16 == 0);
 }
 
 const char* tile_variant_name(int variant)
@@ -425,7 +618,7 @@ hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partia
     case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, s);
     case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, s);
     case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, s);
-    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, s);
+    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4, true>(g, ksplit, partial, s);
     default: return hipErrorInvalidValue;
     }
 }
