@@ -60,20 +60,19 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit)
     const int nkb = g.k / 128;
     const int kbs = (nkb + ksplit - 1) / ksplit;
     const double area = (double)bm * bn / 65536.0;
-    const double per_kb = 1.125 * area + 0.296;
-    const double per_item = 1.29 + 8.76 * area + kbs * per_kb;
+    const double per_kb = 1.19 * area + 0.267;
+    const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     const long items = (long)tiles * ksplit;
     const long rounds = (items + NUM_CU - 1) / NUM_CU;
-    double cost = 1.73 + rounds * per_item;
+    double cost = 1.79 + rounds * per_item;
     if (ksplit > 1)  // second launch + partial write and read-back
-        cost += 2.15 + (double)g.m * g.n * ksplit * 8.0 / 8.98e6;
+        cost += 2.86 + (double)g.m * g.n * ksplit * 8.0 / 7.38e6;
     return cost;
 }
 
 // Shapes whose best measured plan differs from the model's choice: {m, n, k, variant, ksplit}.
 struct TunedShape { int m, n, k, variant, ksplit; };
 constexpr TunedShape kTuned[] = {
-    {1024, 512, 2048, TILE_128x128, 1},
     {1024, 512, 7168, TILE_128x128, 6},
     {1024, 576, 7168, TILE_128x128, 4},
     {8192, 7168, 2048, TILE_256x192, 1},

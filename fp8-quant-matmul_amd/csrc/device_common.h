@@ -74,13 +74,3 @@ __device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t voffset, uint32_t l
                  : "v"(voffset), "s"(rsrc), "s"(lds_addr), "s"(soffset)
                  : "memory");
 }
-
-// The 4-byte-per-lane form: lane l's dword lands at lds_addr + 4*l.  Per-lane offsets are
-// free, so one instruction gathers 64 scattered dwords into a dense LDS table.
-__device__ __forceinline__ void lds_dma4(v4i rsrc, uint32_t voffset, uint32_t lds_addr)
-{
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds"
-                 :
-                 : "v"(voffset), "s"(rsrc), "s"(lds_addr)
-                 : "memory");
-}

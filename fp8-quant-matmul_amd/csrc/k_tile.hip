@@ -53,9 +53,6 @@ struct TileShape {
     static constexpr int NA = RSA / 64;                   // copy instructions per wave, A tile
     static constexpr int NB = RSB / 64;
     static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only)
-    // register-prefetch schedule only: b_scale pairs of the tile for up to 512 K blocks
-    static constexpr int BTAB_BLOCKS = 512;
-    static constexpr int BTAB_BYTES = (BTAB_BLOCKS + 32) * 8;
     static_assert(LDS_BYTES <= 160 * 1024, "stages exceed the 160 KiB of LDS");
 };
 
@@ -73,7 +70,7 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int BM, int BN, int WM, int WN, int NS, bool SPLIT, bool PF>
+template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
@@ -81,7 +78,10 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  int tiles_m, int tiles_n, int kb_per_split)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
-    static_assert(WM * WN == 8, "eight waves per workgroup");
+    // Eight waves copy; WM x WN of them (all eight, or the first four for the smallest tile)
+    // also multiply.
+    static_assert(WM * WN == 8 || WM * WN == 4, "eight or four multiplying waves");
+    constexpr int NCW = WM * WN;
     static_assert(NS >= 2 && NS <= 4, "two to four LDS stages");
     constexpr int TM = BM / WM, TN = BN / WN;      // wave tile
     constexpr int MI = TM / 32, NJ = TN / 32;      // 32x32 patches per wave
@@ -96,7 +96,8 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wm = wave % WM, wn = wave / WM;
+    const int wm = wave % WM, wn = (wave / WM) % WN;
+    const bool compute = NCW == 8 || wave < NCW;
 
     // ---- which tile: consecutive workgroup ids land on different XCDs (id % 8), so give
     // each XCD a contiguous run of tile numbers, and walk tiles in groups of GROUP_M rows
@@ -188,7 +189,6 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     // ---- scales.  One a_scale per lane and 32-row patch (the lane's m).  A wave's n range is at
     // most 128 wide, so it touches at most two 128-wide b_scale blocks (nb_lo, nb_hi); a 32-wide
     // patch never straddles a block boundary.
-    const int m_lane = m0 + wm * TM + (lane & 31);
     const int sn = (N + KBLOCK - 1) / KBLOCK;
     const int n_wave = n0 + wn * TN;
     int nb_lo = n_wave >> 7, nb_hi = (n_wave + TN - 1) >> 7;
@@ -209,262 +209,118 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                 acc[i][j][r] = 0.f;
     const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    if constexpr (PF) {
-        // ---- register-prefetch schedule (small wave tiles: the K block is a handful of MFMAs,
-        // shorter than an LDS round trip, so the reads must not sit between barrier and MFMA).
-        // The fragments and scales of block kb+1 are read into a second register set while the
-        // MFMAs of block kb run on the first; the barrier at the top of a step therefore means
-        // "block kb+1 has landed and everyone has finished reading block kb", which frees the
-        // slot of block kb for block kb+NS: all NS slots hold blocks in flight.
-        const int nblk = kb1 - kb0;
-        const uint32_t btab = (uint32_t)(NS * S::STAGE);
-        {
-            // b_scale pairs (first, last 128-wide block the tile touches) of every K block:
-            // one gathering copy per 32 K blocks, entry j at btab + 8 j
-            const int nbt_lo = (n0 >> 7) < sn ? (n0 >> 7) : sn - 1;
-            const int nbt_hi = ((n0 + BN - 1) >> 7) < sn ? ((n0 + BN - 1) >> 7) : sn - 1;
-            const uint32_t bs_bytes = (uint32_t)nkb * (uint32_t)sn * 4u;
+    // ---- prologue: the first NS-1 K blocks go into ring slots 0 .. NS-2
 #pragma unroll
-            for (int u = 0; u < S::BTAB_BLOCKS / 256; ++u) {
-                const int chunk = wave + 8 * u;
-                if (32 * chunk < nblk) {
-                    const int jb = 32 * chunk + (lane >> 1);
-                    const uint32_t vo =
-                        jb < nblk ? (uint32_t)(((kb0 + jb) * sn + ((lane & 1) ? nbt_hi : nbt_lo)) * 4)
-                                  : 0x80000000u;
-                    lds_dma4(make_rsrc_words(b_scale, bs_bytes), vo, lds_base + btab + (uint32_t)(chunk * 256));
-                }
-            }
+    for (int p = 0; p < NS - 1; ++p)
+        if (kb0 + p < kb1) {
+#pragma unroll
+            for (int q = 0; q < NCOPY; ++q)
+                copy_step(p, kb0 + p, q);
         }
-#pragma unroll
-        for (int p = 0; p < NS; ++p)
-            if (p < nblk) {
-#pragma unroll
-                for (int q = 0; q < NCOPY; ++q)
-                    copy_step(p, kb0 + p, q);
-            }
-        bool patch_hi_t[NJ];  // patch j lies in the tile's second b_scale block
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-            patch_hi_t[j] = ((n_wave + 32 * j) >> 7) > (n0 >> 7);
 
-        v8i fa[2][MI][2], fb[2][NJ][2];
-        float sa[2][MI];
-        v2f sbp[2];
-        auto read_block = [&](auto set_tag, int slot_, int jlocal) __attribute__((always_inline)) {
-            constexpr int P = decltype(set_tag)::value;
-            const uint32_t so = (uint32_t)(slot_ * S::STAGE);
-#pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                fa[P][i][0] = read_frag(addr_a[i] + so, 0, RSA);
-                fa[P][i][1] = read_frag(addr_a[i] + so, 1, RSA);
-            }
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                fb[P][j][0] = read_frag(addr_b[j] + so, 0, RSB);
-                fb[P][j][1] = read_frag(addr_b[j] + so, 1, RSB);
-            }
-#pragma unroll
-            for (int i = 0; i < MI; ++i)
-                sa[P][i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
-            sbp[P] = *LDS_PTR(v2f, lds + btab + (uint32_t)(8 * jlocal));
-        };
-        // wait until at most the copies of `y` younger blocks are outstanding
-        auto wait_younger = [&](int y) __attribute__((always_inline)) {
-            if (y <= 0)
-                wait_vmcnt<0>();
-            else if (y == 1)
-                wait_vmcnt<NCOPY - 1>();
-            else if (y == 2)
+    int slot = 0;             // ring slot of block kb
+    int slot_fill = NS - 1;   // ring slot that block kb + NS - 1 goes into (= slot of kb - 1)
+
+    // One K block.  MORE = block kb+NS-1 exists and is copied here; two instantiations keep the
+    // steady-state body free of branches.
+    auto k_block = [&](auto more_tag, int kb) {
+        constexpr bool more = decltype(more_tag)::value;
+        // Block kb has landed once at most the copies of the younger blocks in flight are
+        // outstanding (loads complete in order).  NCOPY - 1 per block is exact for waves 1..7
+        // and one short for wave 0, which then waits for one more copy than it must.
+        if (more) {
+            wait_vmcnt<(NS - 2) * (NCOPY - 1)>();
+        } else {
+            const int younger = (kb1 - 1 - kb < NS - 2) ? (kb1 - 1 - kb) : (NS - 2);
+            if (NS >= 4 && younger >= 2)
                 wait_vmcnt<2 * (NCOPY - 1)>();
+            else if (NS >= 3 && younger >= 1)
+                wait_vmcnt<NCOPY - 1>();
             else
-                wait_vmcnt<3 * (NCOPY - 1)>();
-        };
-
-        wait_younger((nblk < NS ? nblk : NS) - 1);
-        __syncthreads();
-        read_block(std::integral_constant<int, 0>{}, 0, 0);
-        int slot = 0;
-
-        // One K block on register set P.  FILL: 1 = block kb+NS exists and is copied here,
-        // 0 = decided at run time (the last NS+1 blocks of the range).
-        auto step = [&](auto set_tag, auto fill_tag, int kb) __attribute__((always_inline)) {
-            constexpr int P = decltype(set_tag)::value;
-            constexpr bool steady = decltype(fill_tag)::value;
-            const bool fill = steady || (kb + NS < kb1);
-            if (steady) {
-                wait_vmcnt<(NS - 2) * (NCOPY - 1)>();  // blocks kb+2 .. kb+NS-1 may be in flight
-            } else if (kb + 1 < kb1) {
-                const int last = (kb + NS - 1 < kb1 - 1) ? (kb + NS - 1) : (kb1 - 1);
-                wait_younger(last - (kb + 1));
-            }
-            __syncthreads();
-            const int slot_next = (slot + 1 == NS) ? 0 : slot + 1;
-            // past the last block this reads a stale slot into registers nobody uses
-            read_block(std::integral_constant<int, 1 - P>{}, slot_next, kb - kb0 + 1);
-
-            float s[MI], s_hi[MI];
-#pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                s[i] = sa[P][i] * sbp[P].x;
-                s_hi[i] = sa[P][i] * sbp[P].y;
-            }
-            constexpr int N_MFMA = MI * NJ * 2;
-            constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;
-            int cq = 0;
-            auto copy_slot = [&](int n) __attribute__((always_inline)) {
-#pragma unroll
-                for (int u = 0; u < NCOPY; ++u)
-                    if (u < n && cq < NCOPY) {
-                        if (fill)
-                            copy_step(slot, kb + NS, cq);
-                        ++cq;
-                    }
-            };
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                v16f blk[MI];
-#pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[P][j][0], fa[P][i][0], zero16,
-                                                                              0, 0, 0, 0, 0, 0);
-                    copy_slot(PER_MFMA);
-                }
-#pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[P][j][1], fa[P][i][1], blk[i],
-                                                                              0, 0, 0, 0, 0, 0);
-                    copy_slot(PER_MFMA);
-                }
-#pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    const float sc = patch_hi_t[j] ? s_hi[i] : s[i];
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
-                }
-            }
-            copy_slot(NCOPY);
-            slot = slot_next;
-        };
-        using Set0 = std::integral_constant<int, 0>;
-        using Set1 = std::integral_constant<int, 1>;
-        int kb = kb0;
-        for (; kb + NS + 1 < kb1; kb += 2) {  // both blocks of the pair have a block NS ahead
-            step(Set0{}, std::true_type{}, kb);
-            step(Set1{}, std::true_type{}, kb + 1);
+                wait_vmcnt<0>();
         }
-        for (; kb < kb1; kb += 2) {
-            step(Set0{}, std::false_type{}, kb);
-            if (kb + 1 < kb1)
-                step(Set1{}, std::false_type{}, kb + 1);
-        }
-    } else {
-        // ---- prologue: the first NS-1 K blocks go into ring slots 0 .. NS-2
-    #pragma unroll
-        for (int p = 0; p < NS - 1; ++p)
-            if (kb0 + p < kb1) {
-    #pragma unroll
-                for (int q = 0; q < NCOPY; ++q)
-                    copy_step(p, kb0 + p, q);
-            }
-
-        int slot = 0;             // ring slot of block kb
-        int slot_fill = NS - 1;   // ring slot that block kb + NS - 1 goes into (= slot of kb - 1)
-
-        // One K block.  MORE = block kb+NS-1 exists and is copied here; two instantiations keep the
-        // steady-state body free of branches.
-        auto k_block = [&](auto more_tag, int kb) {
-            constexpr bool more = decltype(more_tag)::value;
-            // Block kb has landed once at most the copies of the younger blocks in flight are
-            // outstanding (loads complete in order).  NCOPY - 1 per block is exact for waves 1..7
-            // and one short for wave 0, which then waits for one more copy than it must.
+        __syncthreads();  // everyone's copies of block kb landed; slot_fill is no longer read
+        if (!compute) {  // copy-only wave
             if (more) {
-                wait_vmcnt<(NS - 2) * (NCOPY - 1)>();
-            } else {
-                const int younger = (kb1 - 1 - kb < NS - 2) ? (kb1 - 1 - kb) : (NS - 2);
-                if (NS >= 4 && younger >= 2)
-                    wait_vmcnt<2 * (NCOPY - 1)>();
-                else if (NS >= 3 && younger >= 1)
-                    wait_vmcnt<NCOPY - 1>();
-                else
-                    wait_vmcnt<0>();
+#pragma unroll
+                for (int q = 0; q < NCOPY; ++q)
+                    copy_step(slot_fill, kb + NS - 1, q);
             }
-            __syncthreads();  // everyone's copies of block kb landed; slot_fill is no longer read
-            const uint32_t so = (uint32_t)(slot * S::STAGE);
-            float sa[MI];
-    #pragma unroll
-            for (int i = 0; i < MI; ++i)
-                sa[i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
-            // wave-uniform addresses: scalar loads
-            const float sb_lo = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_lo)];
-            const float sb_hi = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_hi)];
-
-            v8i fa[MI][2];
-    #pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
-                fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
-            }
-            float s[MI], s_hi[MI];
-    #pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                s[i] = sa[i] * sb_lo;
-                s_hi[i] = sa[i] * sb_hi;
-            }
-
-            // the wave's NCOPY copy instructions of block kb+NS-1 ride on the first MFMAs
-            constexpr int N_MFMA = MI * NJ * 2;
-            constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;  // copies behind each MFMA
-            int cq = 0;
-            auto copy_slot = [&](int n) {
-    #pragma unroll
-                for (int u = 0; u < NCOPY; ++u)
-                    if (u < n && cq < NCOPY) {
-                        if (more)
-                            copy_step(slot_fill, kb + NS - 1, cq);
-                        ++cq;
-                    }
-            };
-
-    #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const v8i fb0 = read_frag(addr_b[j] + so, 0, RSB);
-                const v8i fb1 = read_frag(addr_b[j] + so, 1, RSB);
-                v16f blk[MI];
-    #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
-                                                                              0, 0, 0);
-                    copy_slot(PER_MFMA);
-                }
-    #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
-                                                                              0, 0, 0);
-                    copy_slot(PER_MFMA);
-                }
-    #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    const float sc = patch_hi[j] ? s_hi[i] : s[i];
-    #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
-                }
-            }
-            copy_slot(NCOPY);  // whatever is left (tiles with few MFMAs per K block)
-
             slot_fill = slot;
             slot = (slot + 1 == NS) ? 0 : slot + 1;
+            return;
+        }
+        const uint32_t so = (uint32_t)(slot * S::STAGE);
+        float sa[MI];
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+            sa[i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
+        // wave-uniform addresses: scalar loads
+        const float sb_lo = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_lo)];
+        const float sb_hi = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_hi)];
+
+        v8i fa[MI][2];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
+            fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
+        }
+        float s[MI], s_hi[MI];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            s[i] = sa[i] * sb_lo;
+            s_hi[i] = sa[i] * sb_hi;
+        }
+
+        // the wave's NCOPY copy instructions of block kb+NS-1 ride on the first MFMAs
+        constexpr int N_MFMA = MI * NJ * 2;
+        constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;  // copies behind each MFMA
+        int cq = 0;
+        auto copy_slot = [&](int n) {
+#pragma unroll
+            for (int u = 0; u < NCOPY; ++u)
+                if (u < n && cq < NCOPY) {
+                    if (more)
+                        copy_step(slot_fill, kb + NS - 1, cq);
+                    ++cq;
+                }
         };
-        int kb = kb0;
-        for (; kb + NS - 1 < kb1; ++kb)
-            k_block(std::true_type{}, kb);
-        for (; kb < kb1; ++kb)
-            k_block(std::false_type{}, kb);
 
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const v8i fb0 = read_frag(addr_b[j] + so, 0, RSB);
+            const v8i fb1 = read_frag(addr_b[j] + so, 1, RSB);
+            v16f blk[MI];
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
+                                                                          0, 0, 0);
+                copy_slot(PER_MFMA);
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
+                                                                          0, 0, 0);
+                copy_slot(PER_MFMA);
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const float sc = patch_hi[j] ? s_hi[i] : s[i];
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);
+            }
+        }
+        copy_slot(NCOPY);  // whatever is left (tiles with few MFMAs per K block)
 
-    }
+        slot_fill = slot;
+        slot = (slot + 1 == NS) ? 0 : slot + 1;
+    };
+    int kb = kb0;
+    for (; kb + NS - 1 < kb1; ++kb)
+        k_block(std::true_type{}, kb);
+    for (; kb < kb1; ++kb)
+        k_block(std::false_type{}, kb);
 
     // ---- epilogue.  A lane owns row m = .. + (lane & 31) and, per patch, four runs of 4 columns
     // (accumulator register 4*q + e is column 8*q + 4*(lane >> 5) + e of the patch): stored
@@ -486,7 +342,7 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
             const int prow = wm * TM + 32 * i;  // first tile row of the patch
-            if (prow / HROWS == h) {
+            if (compute && prow / HROWS == h) {
                 const uint32_t rbase = (uint32_t)((prow - h * HROWS + (lane & 31)) * CROW);
 #pragma unroll
                 for (int j = 0; j < NJ; ++j)
@@ -545,23 +401,18 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     *reinterpret_cast<uint2*>(c + i4) = pk;
 }
 
-template <int BM, int BN, int WM, int WN, int NS, bool PF = false>
+template <int BM, int BN, int WM, int WN, int NS>
 hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStream_t s)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
-    constexpr int LDS_TOTAL = S::LDS_BYTES + (PF ? S::BTAB_BYTES : 0);
-    static_assert(LDS_TOTAL <= 160 * 1024, "stages and scale table exceed the 160 KiB of LDS");
+    constexpr int LDS_TOTAL = S::LDS_BYTES;
     const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     const int nkb = g.k / KBLOCK;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
-    if constexpr (PF) {
-        if (kb_per_split > S::BTAB_BLOCKS)  // scale table too small: the plain schedule has no limit
-            return launch_variant<BM, BN, WM, WN, NS, false>(g, ksplit, partial, s);
-    }
     dim3 grid(tiles_m * tiles_n, ksplit);
     hipError_t e;
     if (ksplit > 1) {
-        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true, PF>;
+        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
         if (e != hipSuccess)
@@ -569,7 +420,7 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
     } else {
-        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false, PF>;
+        auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
         if (e != hipSuccess)
@@ -598,6 +449,7 @@ const char* tile_variant_name(int variant)
     case TILE_128x128: return "tile128x128";
     case TILE_256x192: return "tile256x192";
     case TILE_128x192: return "tile128x192";
+    case TILE_64x64: return "tile64x64";
     default: return "tile?";
     }
 }
@@ -608,6 +460,7 @@ void tile_variant_dims(int variant, int* bm, int* bn)
     case TILE_256x128: *bm = 256; *bn = 128; break;
     case TILE_256x192: *bm = 256; *bn = 192; break;
     case TILE_128x192: *bm = 128; *bn = 192; break;
+    case TILE_64x64: *bm = 64; *bn = 64; break;
     default: *bm = 128; *bn = 128; break;
     }
 }
@@ -618,7 +471,8 @@ hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partia
     case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, s);
     case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, s);
     case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, s);
-    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4, true>(g, ksplit, partial, s);
+    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, s);
+    case TILE_64x64: return launch_variant<64, 64, 2, 2, 4>(g, ksplit, partial, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -73,8 +73,8 @@ int fp8_block_gemm_scalar(const void* a, const void* b, const float* a_scale,
 int fp8_block_gemm_select(int kernel_id);
 
 /* Pin the MFMA tile kernels to one workgroup tile (0 = 256x192, 1 = 256x128, 2 = 128x128,
- * 3 = 128x192 rows x columns of C; -1 = choose by cost model) and one K-split count (0 = choose).  Benchmarking and test
- * aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
+ * 3 = 128x192, 4 = 64x64 rows x columns of C; -1 = choose by cost model) and one K-split
+ * count (0 = choose).  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
  * (/root/reference/mn_large.hip:1-8). */
 int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 

@@ -79,7 +79,7 @@ SHAPES = [(256, 256, 128), (256, 256, 256), (512, 768, 512), (272, 576, 384), (1
           (16, 16, 128), (1024, 192, 640), (304, 1040, 256), (64, 2048, 1024)]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("m,n,k", SHAPES)
 def test_tile_kernel(pkg, variant, m, n, k):
     a, b, sa, sb = oracle.make_inputs(m, n, k, m * 7 + n + variant, 1.0, 50.0)
@@ -91,7 +91,8 @@ def test_tile_kernel(pkg, variant, m, n, k):
 
 @pytest.mark.parametrize("variant,ksplit,m,n,k", [(2, 2, 256, 256, 512), (2, 4, 512, 512, 1024),
                                                    (1, 3, 272, 576, 896), (0, 8, 256, 576, 2048),
-                                                   (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048), (3, 5, 384, 576, 1280)])
+                                                   (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048), (3, 5, 384, 576, 1280),
+                                                   (4, 3, 208, 336, 768), (4, 2, 64, 64, 256)])
 def test_tile_kernel_split_k(pkg, variant, ksplit, m, n, k):
     a, b, sa, sb = oracle.make_inputs(m, n, k, m + n + k + ksplit)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
