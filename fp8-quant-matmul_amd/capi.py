@@ -60,6 +60,8 @@ def lib():
     L.fp8_block_gemm_select.argtypes = [i]
     L.fp8_block_gemm_force_config.restype = i
     L.fp8_block_gemm_force_config.argtypes = [i, i]
+    L.fp8_block_gemm_set_persistent.restype = i
+    L.fp8_block_gemm_set_persistent.argtypes = [i]
     L.fp8_block_gemm_plan.restype = i
     L.fp8_block_gemm_plan.argtypes = [i, i, i, C.c_char_p, sz]
     L.fp8_block_gemm_last_kernel.restype = C.c_char_p
@@ -127,6 +129,11 @@ def select(kernel_id):
 
 def force_config(tile_variant=-1, ksplit=0):
     _check(lib().fp8_block_gemm_force_config(tile_variant, ksplit), "fp8_block_gemm_force_config")
+
+
+def set_persistent(mode=-1):
+    """-1: persistent tile kernel when tiles outnumber the CUs, 0: never, 1: whenever possible"""
+    _check(lib().fp8_block_gemm_set_persistent(mode), "fp8_block_gemm_set_persistent")
 
 
 def plan(m, n, k):

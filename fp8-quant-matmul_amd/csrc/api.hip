@@ -19,6 +19,7 @@ constexpr int NUM_CU = 256;
 std::atomic<int> g_selected{FP8GEMM_KERNEL_AUTO};
 std::atomic<int> g_force_variant{-1};
 std::atomic<int> g_force_ksplit{0};
+std::atomic<int> g_persistent{-1};  // -1 = when tiles outnumber the CUs, 0 = never, 1 = whenever possible
 thread_local const char* t_last_kernel = "none";
 thread_local char t_name_buf[64];
 
@@ -32,6 +33,7 @@ struct Plan {
     int family;   // FP8GEMM_KERNEL_*
     int variant;  // TileVariant for the tile families
     int ksplit;
+    bool persistent = false;  // tile families, ksplit == 1: workgroups walk through the tiles
 };
 
 int validate(const void* a, const void* b, const float* as, const float* bs, const void* c, int m,
@@ -78,6 +80,19 @@ constexpr TunedShape kTuned[] = {
     {8192, 7168, 2048, TILE_256x192, 1},
 };
 
+// A persistent launch pays off when a CU gets more than one tile.
+void decide_persistent(const GemmArgs& g, Plan& p)
+{
+    p.persistent = false;
+    const int mode = g_persistent.load();
+    if (mode == 0 || p.ksplit != 1 || !tile_persistent_supports(g, p.variant))
+        return;
+    int bm, bn;
+    tile_variant_dims(p.variant, &bm, &bn);
+    const long tiles = (long)((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
+    p.persistent = mode == 1 || tiles > NUM_CU;
+}
+
 Plan make_plan(const GemmArgs& g, int selected)
 {
     Plan p{FP8GEMM_KERNEL_SCALAR, 0, 1};
@@ -107,6 +122,7 @@ Plan make_plan(const GemmArgs& g, int selected)
                 p.family = t.ksplit > 1 ? FP8GEMM_KERNEL_SPLITK : FP8GEMM_KERNEL_LARGE;
                 p.variant = t.variant;
                 p.ksplit = t.ksplit;
+                decide_persistent(g, p);
                 return p;
             }
     double best = 1e300;
@@ -137,6 +153,8 @@ Plan make_plan(const GemmArgs& g, int selected)
     }
     if (best == 1e300)
         p.family = -1;
+    else
+        decide_persistent(g, p);
     return p;
 }
 
@@ -221,10 +239,15 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
             if (!ws)
                 return err;
         }
-        e = launch_tile(g, p.variant, p.ksplit, ws, stream);
-        if (e == hipSuccess && p.ksplit > 1)
-            e = launch_splitk_reduce(g, p.ksplit, ws, stream);
-        snprintf(t_name_buf, sizeof(t_name_buf), "%s_k%d", tile_variant_name(p.variant), p.ksplit);
+        if (p.persistent) {
+            e = launch_tile_persistent(g, p.variant, NUM_CU, stream);
+        } else {
+            e = launch_tile(g, p.variant, p.ksplit, ws, stream);
+            if (e == hipSuccess && p.ksplit > 1)
+                e = launch_splitk_reduce(g, p.ksplit, ws, stream);
+        }
+        snprintf(t_name_buf, sizeof(t_name_buf), "%s_k%d%s", tile_variant_name(p.variant), p.ksplit,
+                 p.persistent ? "_persistent" : "");
         t_last_kernel = t_name_buf;
         break;
     }
@@ -273,6 +296,14 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit)
     return FP8GEMM_OK;
 }
 
+int fp8_block_gemm_set_persistent(int mode)
+{
+    if (mode < -1 || mode > 1)
+        return FP8GEMM_E_KERNEL;
+    g_persistent.store(mode);
+    return FP8GEMM_OK;
+}
+
 const char* fp8_block_gemm_last_kernel(void) { return t_last_kernel; }
 
 int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap)
@@ -292,7 +323,8 @@ int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap)
     else if (p.family == FP8GEMM_KERNEL_SKINNY)
         snprintf(name, cap, "skinny_k%d", p.ksplit);
     else
-        snprintf(name, cap, "%s_k%d", tile_variant_name(p.variant), p.ksplit);
+        snprintf(name, cap, "%s_k%d%s", tile_variant_name(p.variant), p.ksplit,
+                 p.persistent ? "_persistent" : "");
     return FP8GEMM_OK;
 }
 

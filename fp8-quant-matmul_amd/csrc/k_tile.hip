@@ -29,46 +29,11 @@
 //     and holds every wave back from its LDS reads).
 //
 // Work decomposition: grid.x = tiles (XCD-aware order), grid.y = K splits.
-#include "device_common.h"
-#include "launchers.h"
-
-#include <type_traits>
+#include "tile_common.h"
 
 namespace fp8gemm {
 
 namespace {
-
-constexpr int NTHREADS = 512;
-constexpr int GROUP_M = 8;  // tile rows per L2 locality group
-
-template <int BM, int BN, int WM, int WN, int NS>
-struct TileShape {
-    static constexpr int RSA = BM > 128 ? 256 : 128;  // LDS bytes per k-row of the A tile
-    static constexpr int RSB = BN > 128 ? 256 : 128;
-    static constexpr int MAT_A = KBLOCK * RSA;
-    static constexpr int MAT_B = KBLOCK * RSB;
-    static constexpr int SCALE_OFF = MAT_A + MAT_B;       // BM a_scale floats
-    static constexpr int STAGE = MAT_A + MAT_B + 1024;
-    static constexpr int LDS_BYTES = NS * STAGE;
-    static constexpr int NA = RSA / 64;                   // copy instructions per wave, A tile
-    static constexpr int NB = RSB / 64;
-    static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only)
-    static_assert(LDS_BYTES <= 160 * 1024, "stages exceed the 160 KiB of LDS");
-};
-
-// chunk swizzle of row r (0..7 within an 8-row group) for a row stride of RS bytes
-template <int RS>
-__device__ __forceinline__ int row_swizzle(int r)
-{
-    return RS == 256 ? 2 * (r & 7) : 2 * ((r >> 1) & 3);
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
 
 template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
 __global__ void __launch_bounds__(NTHREADS)
@@ -123,16 +88,16 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     // NA*w .. NA*w+NA-1 of the A tile and likewise of B.  A lane writes chunk position p of
     // row r and therefore fetches column chunk p ^ swizzle(r).  Chunks outside the tile or the
     // matrix get an out-of-range offset: the buffer load then writes zeros and reads nothing.
-    uint32_t voff_a[NA], voff_b[NB];
+    uint32_t voff_a[S::NVA], voff_b[S::NVB];
 #pragma unroll
-    for (int q = 0; q < NA; ++q) {
+    for (int q = 0; q < S::NVA; ++q) {
         const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
         const int cc = (RSA == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSA>(r & 7);
         const bool ok = (16 * cc < BM) && (m0 + 16 * cc < M);
         voff_a[q] = ok ? (uint32_t)(r * M + m0 + 16 * cc) : 0x80000000u;
     }
 #pragma unroll
-    for (int q = 0; q < NB; ++q) {
+    for (int q = 0; q < S::NVB; ++q) {
         const int r = RSB == 256 ? (NB * wave + q) * 4 + (lane >> 4) : (NB * wave + q) * 8 + (lane >> 3);
         const int cc = (RSB == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSB>(r & 7);
         const bool ok = (16 * cc < BN) && (n0 + 16 * cc < N);
@@ -150,11 +115,12 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     auto copy_step = [&](int slot, int kb, int q) __attribute__((always_inline)) {
         const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
         if (q < NA) {
-            lds_dma16(rsrc_a, voff_a[q], stage + (uint32_t)((NA * wave + q) * 1024),
-                      (uint32_t)kb * KBLOCK * (uint32_t)M);
+            lds_dma16(rsrc_a, voff_a[S::template voff_index<RSA>(q)], stage + (uint32_t)((NA * wave + q) * 1024),
+                      (uint32_t)(kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)M);
         } else if (q < NA + NB) {
-            lds_dma16(rsrc_b, voff_b[q - NA], stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
-                      (uint32_t)kb * KBLOCK * (uint32_t)N);
+            lds_dma16(rsrc_b, voff_b[S::template voff_index<RSB>(q - NA)],
+                      stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
+                      (uint32_t)(kb * KBLOCK + S::template extra_rows<RSB>(q - NA)) * (uint32_t)N);
         } else if (wave == 0) {
             lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)kb * (uint32_t)M * 4u);
         }

@@ -1,0 +1,379 @@
+// Persistent form of the MFMA tile kernel for shapes with more tiles than compute units.
+//
+// The plain kernel (k_tile.hip) runs one tile per workgroup: with one workgroup per CU (the LDS
+// ring fills the CU) every round of 256 tiles pays the launch of a new workgroup, an empty
+// ring (one global round trip before the first MFMA) and an output burst during which no MFMA
+// runs.  Here a workgroup walks through its tiles itself and the ring never drains: the K
+// blocks of all its tiles form one stream, the copies for block g+NS-1 of the stream are
+// issued while block g is multiplied, also across a tile boundary, so the first blocks of
+// the next tile land while the finished tile is converted and stored.
+//
+// The finished tile cannot use the whole ring as its staging area (NS-1 slots hold the next
+// tile's blocks): it leaves in pieces of PR rows through the one slot whose block was
+// multiplied last.
+//
+// Data path, LDS layout, MFMA orientation and scale folding are those of k_tile.hip
+// (successor of in_smem_kernel, /root/reference/mn_large.hip:11-128; the reference lists a
+// persistent kernel that overlaps the epilogue with the next tile as future work,
+// /root/reference/README.md:29).
+#include "tile_common.h"
+
+namespace fp8gemm {
+
+namespace {
+
+template <int BM, int BN, int WM, int WN, int NS, int PR>
+__global__ void __launch_bounds__(NTHREADS)
+tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                            const float* __restrict__ a_scale, const float* __restrict__ b_scale,
+                            uint16_t* __restrict__ c, int M, int N, int K, int tiles_m, int tiles_n)
+{
+    using S = TileShape<BM, BN, WM, WN, NS>;
+    static_assert(WM * WN == 8, "eight waves per workgroup");
+    static_assert(NS >= 2 && NS <= 4, "two to four LDS stages");
+    constexpr int TM = BM / WM, TN = BN / WN;
+    constexpr int MI = TM / 32, NJ = TN / 32;
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && TN <= 128 && BM <= 256 && BN <= 256, "wave tile");
+    constexpr int RSA = S::RSA, RSB = S::RSB, NA = S::NA, NB = S::NB, NCOPY = S::NCOPY;
+    constexpr int CROW = BN * 2 + 8;          // staging bytes per tile row (conflict-free writes)
+    static_assert(PR % 32 == 0 && BM % PR == 0, "a piece is a whole number of 32-row patches");
+    static_assert(PR * CROW <= S::STAGE, "a piece must fit one ring slot");
+    constexpr int CPR = BN / 8;               // 16-byte chunks per tile row
+    constexpr int CHUNKS = PR * CPR;
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    auto lds = LDS_PTR(uint8_t, smem);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+
+    // ---- this workgroup's tiles.  Workgroup ids go round the 8 XCDs (id % 8); each XCD owns
+    // a contiguous run of the tile order (groups of GROUP_M tile rows, as in k_tile.hip) and
+    // its workgroups take the run's tiles in turn, so that the tiles an XCD works on at any
+    // moment are neighbours and share A and B panels in its L2.
+    const int T = tiles_m * tiles_n;
+    const int pid = blockIdx.x, per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
+    const int xcd = pid & 7, q8 = T >> 3, r8 = T & 7;
+    const int run0 = xcd * q8 + (xcd < r8 ? xcd : r8);
+    const int run_len = q8 + (xcd < r8 ? 1 : 0);
+    const int li = pid >> 3;
+    const int n_my = li < run_len ? (run_len - li + per_xcd - 1) / per_xcd : 0;
+    if (n_my == 0)
+        return;
+    const int per_group = GROUP_M * tiles_n;
+    auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {
+        const int logical = run0 + li + j * per_xcd;
+        const int group = logical / per_group;
+        const int first_m = group * GROUP_M;
+        const int gsz = (tiles_m - first_m < GROUP_M) ? (tiles_m - first_m) : GROUP_M;
+        const int in_group = logical - group * per_group;
+        m0 = (first_m + in_group % gsz) * BM;
+        n0 = (in_group / gsz) * BN;
+    };
+
+    const int nkb = K / KBLOCK;
+    const int sn = (N + KBLOCK - 1) / KBLOCK;
+    const uint32_t a_bytes = (uint32_t)M * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
+    const uint32_t as_bytes = (uint32_t)nkb * (uint32_t)M * 4u;
+    const v4i rsrc_a = make_rsrc_words(a, a_bytes), rsrc_b = make_rsrc_words(b, b_bytes);
+    const v4i rsrc_s = make_rsrc_words(a_scale, as_bytes);
+
+    // ---- the copy stream: K block f_kb of this workgroup's tile number f_tile is the next one
+    // to be copied.  Per-lane offsets (copy plan of k_tile.hip) belong to that tile.
+    uint32_t voff_a[S::NVA], voff_b[S::NVB], voff_s;
+    int f_tile = 0, f_kb = 0;
+    int fill_left = n_my * nkb;  // blocks not yet copied
+    auto fill_setup = [&](int j) __attribute__((always_inline)) {
+        int m0, n0;
+        tile_origin(j, m0, n0);
+#pragma unroll
+        for (int q = 0; q < S::NVA; ++q) {
+            const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
+            const int cc = (RSA == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSA>(r & 7);
+            const bool ok = (16 * cc < BM) && (m0 + 16 * cc < M);
+            voff_a[q] = ok ? (uint32_t)(r * M + m0 + 16 * cc) : 0x80000000u;
+        }
+#pragma unroll
+        for (int q = 0; q < S::NVB; ++q) {
+            const int r = RSB == 256 ? (NB * wave + q) * 4 + (lane >> 4) : (NB * wave + q) * 8 + (lane >> 3);
+            const int cc = (RSB == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSB>(r & 7);
+            const bool ok = (16 * cc < BN) && (n0 + 16 * cc < N);
+            voff_b[q] = ok ? (uint32_t)(r * N + n0 + 16 * cc) : 0x80000000u;
+        }
+        voff_s = (4 * lane < BM && m0 + 4 * lane < M) ? (uint32_t)((m0 + 4 * lane) * 4) : 0x80000000u;
+    };
+    // copy instruction q of the stream's next block into ring slot `slot`
+    auto fill_copy = [&](int slot, int q) __attribute__((always_inline)) {
+        const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
+        if (q < NA) {
+            lds_dma16(rsrc_a, voff_a[S::template voff_index<RSA>(q)], stage + (uint32_t)((NA * wave + q) * 1024),
+                      (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)M);
+        } else if (q < NA + NB) {
+            lds_dma16(rsrc_b, voff_b[S::template voff_index<RSB>(q - NA)],
+                      stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
+                      (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSB>(q - NA)) * (uint32_t)N);
+        } else if (wave == 0) {
+            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)f_kb * (uint32_t)M * 4u);
+        }
+    };
+    auto fill_advance = [&]() __attribute__((always_inline)) {
+        --fill_left;
+        if (++f_kb == nkb) {
+            f_kb = 0;
+            ++f_tile;
+            if (fill_left > 0)
+                fill_setup(f_tile);
+        }
+    };
+
+    // ---- LDS read addresses (k_tile.hip): they do not depend on the tile
+    const int g4 = lane >> 4, i16 = lane & 15;
+    uint32_t addr_a[MI], addr_b[NJ];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+        addr_a[i] = (uint32_t)((32 * (g4 >> 1) + (i16 >> 1)) * RSA + (i16 & 1) * 8 +
+                               ((((wm * TM) / 16 + 2 * i + (g4 & 1)) ^ row_swizzle<RSA>(i16 >> 1)) * 16));
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+        addr_b[j] = (uint32_t)(S::MAT_A + (32 * (g4 >> 1) + (i16 >> 1)) * RSB + (i16 & 1) * 8 +
+                               ((((wn * TN) / 16 + 2 * j + (g4 & 1)) ^ row_swizzle<RSB>(i16 >> 1)) * 16));
+    const uint32_t addr_s = S::SCALE_OFF + (uint32_t)((wm * TM + (lane & 31)) * 4);
+    auto read_frag = [&](uint32_t addr, int ks, int rs) __attribute__((always_inline)) -> v8i {
+        const uint32_t base = addr + (uint32_t)(ks * 64 * rs);
+        v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base));
+        v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 8 * rs));
+        v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 16 * rs));
+        v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + base + 24 * rs));
+        return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+    };
+    const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // ---- fill the ring: the first NS-1 blocks of the stream
+    fill_setup(0);
+#pragma unroll
+    for (int p = 0; p < NS - 1; ++p)
+        if (fill_left > 0) {
+#pragma unroll
+            for (int q = 0; q < NCOPY; ++q)
+                fill_copy(p, q);
+            fill_advance();
+        }
+    int slot = 0;            // ring slot of the block being multiplied
+    int slot_fill = NS - 1;  // ring slot the stream's next block goes into
+
+    for (int j = 0; j < n_my; ++j) {
+        int m0, n0;
+        tile_origin(j, m0, n0);
+        const int n_wave = n0 + wn * TN;
+        int nb_lo = n_wave >> 7, nb_hi = (n_wave + TN - 1) >> 7;
+        nb_lo = nb_lo < sn ? nb_lo : sn - 1;
+        nb_hi = nb_hi < sn ? nb_hi : sn - 1;
+        bool patch_hi[NJ];
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj)
+            patch_hi[jj] = ((n_wave + 32 * jj) >> 7) > (n_wave >> 7);
+
+        v16f acc[MI][NJ];
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][jj][r] = 0.f;
+
+        // One K block.  MORE = the stream has a block left to copy (always, except for the last
+        // NS-1 blocks of the last tile).
+        auto k_block = [&](auto more_tag, int kb) __attribute__((always_inline)) {
+            constexpr bool more = decltype(more_tag)::value;
+            // The first NS-1 blocks of a later tile were copied before the previous tile's
+            // epilogue, which waited for them: no wait here, and none that would drag in that
+            // epilogue's stores.  Otherwise at most the younger blocks may be outstanding.
+            const bool landed = j > 0 && kb < NS - 1;
+            if (!landed) {
+                if (more) {
+                    wait_vmcnt<(NS - 2) * (NCOPY - 1)>();
+                } else {
+                    const int younger = (nkb - 1 - kb < NS - 2) ? (nkb - 1 - kb) : (NS - 2);
+                    if (NS >= 4 && younger >= 2)
+                        wait_vmcnt<2 * (NCOPY - 1)>();
+                    else if (NS >= 3 && younger >= 1)
+                        wait_vmcnt<NCOPY - 1>();
+                    else
+                        wait_vmcnt<0>();
+                }
+            }
+            __syncthreads();  // block landed for everyone; slot_fill is no longer read
+            const uint32_t so = (uint32_t)(slot * S::STAGE);
+            float sa[MI];
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+                sa[i] = *LDS_PTR(float, lds + so + addr_s + 128 * i);
+            const float sb_lo = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_lo)];
+            const float sb_hi = b_scale[__builtin_amdgcn_readfirstlane(kb * sn + nb_hi)];
+
+            v8i fa[MI][2];
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
+                fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
+            }
+            float s[MI], s_hi[MI];
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                s[i] = sa[i] * sb_lo;
+                s_hi[i] = sa[i] * sb_hi;
+            }
+            constexpr int N_MFMA = MI * NJ * 2;
+            constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;
+            int cq = 0;
+            auto copy_slot = [&](int n) __attribute__((always_inline)) {
+#pragma unroll
+                for (int u = 0; u < NCOPY; ++u)
+                    if (u < n && cq < NCOPY) {
+                        if (more)
+                            fill_copy(slot_fill, cq);
+                        ++cq;
+                    }
+            };
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) {
+                const v8i fb0 = read_frag(addr_b[jj] + so, 0, RSB);
+                const v8i fb1 = read_frag(addr_b[jj] + so, 1, RSB);
+                v16f blk[MI];
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
+                                                                              0, 0, 0);
+                    copy_slot(PER_MFMA);
+                }
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
+                                                                              0, 0, 0);
+                    copy_slot(PER_MFMA);
+                }
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    const float sc = patch_hi[jj] ? s_hi[i] : s[i];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][jj][r] = fmaf(sc, blk[i][r], acc[i][jj][r]);
+                }
+            }
+            copy_slot(NCOPY);
+            if (more)
+                fill_advance();
+            slot_fill = slot;
+            slot = (slot + 1 == NS) ? 0 : slot + 1;
+        };
+
+        // the host launches this kernel only for nkb >= NS-1: the stream then runs dry in the
+        // last NS-1 blocks of the last tile and nowhere else
+        const int tail = (j + 1 < n_my) ? 0 : NS - 1;
+        int kb = 0;
+        for (; kb < nkb - tail; ++kb)
+            k_block(std::true_type{}, kb);
+        for (; kb < nkb; ++kb)
+            k_block(std::false_type{}, kb);
+
+        // ---- epilogue: bf16, in pieces of PR rows through the ring slot of the block multiplied
+        // last (slot_fill by now; the stream's next copy goes there, but not before the next
+        // K block's barrier), 16 bytes per lane along whole tile rows.  Every copy of the stream
+        // issued so far has to have landed before the first store goes out: the next tile's
+        // first blocks are then known to be there without a wait that would also cover these
+        // stores.
+        wait_vmcnt<0>();
+        const uint32_t staging = (uint32_t)(slot_fill * S::STAGE);
+        __syncthreads();  // every wave has finished reading that slot
+        // opaque copy of the thread id: keeps the address arithmetic below inside the tile loop
+        // (hoisted, it would sit in registers the K loop needs and be spilled)
+        int tid = (int)threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane_e = tid & 63;
+#pragma unroll
+        for (int p = 0; p < BM / PR; ++p) {
+            if (p > 0)
+                __syncthreads();  // the previous piece has been read out
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int prow = wm * TM + 32 * i;
+                if (prow / PR == p) {
+                    const uint32_t rbase = staging + (uint32_t)((prow - p * PR + (lane_e & 31)) * CROW);
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int col = wn * TN + 32 * jj + 8 * q + 4 * (lane_e >> 5);
+                            v2i pk = {(int)pack_bf16x2(acc[i][jj][4 * q], acc[i][jj][4 * q + 1]),
+                                      (int)pack_bf16x2(acc[i][jj][4 * q + 2], acc[i][jj][4 * q + 3])};
+                            *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
+                        }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < (CHUNKS + NTHREADS - 1) / NTHREADS; ++it) {
+                const int idx = it * NTHREADS + tid;
+                const int row = idx / CPR, ch = idx - row * CPR;
+                const int mrow = m0 + p * PR + row;
+                const int ncol = n0 + ch * 8;
+                if (idx < CHUNKS && mrow < M && ncol < N) {
+                    const v2i lo = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16);
+                    const v2i hi = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16 + 8);
+                    *reinterpret_cast<v4i*>(c + (size_t)mrow * N + ncol) = (v4i){lo.x, lo.y, hi.x, hi.y};
+                }
+            }
+        }
+        // the next tile's first K block begins with a barrier: the slot is not written again
+        // before every lane has read its chunks of the last piece
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int NS, int PR>
+hipError_t launch_persistent_variant(const GemmArgs& g, int workgroups, hipStream_t s)
+{
+    using S = TileShape<BM, BN, WM, WN, NS>;
+    constexpr int LDS_TOTAL = S::LDS_BYTES;
+    const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
+    auto kern = tile_gemm_persistent_kernel<BM, BN, WM, WN, NS, PR>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
+    if (e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kern, dim3(workgroups), dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale,
+                       g.b_scale, g.c, g.m, g.n, g.k, tiles_m, tiles_n);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool tile_persistent_supports(const GemmArgs& g, int variant)
+{
+    int stages;
+    switch (variant) {
+    case TILE_256x192: stages = 2; break;
+    case TILE_256x128: stages = 3; break;
+    case TILE_128x192: stages = 3; break;
+    case TILE_128x128: stages = 4; break;
+    default: return false;
+    }
+    return tile_supports(g) && g.k / KBLOCK >= stages - 1;
+}
+
+hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups, hipStream_t s)
+{
+    if (workgroups <= 0 || workgroups % 8 != 0 || !tile_persistent_supports(g, variant))
+        return hipErrorInvalidValue;
+    switch (variant) {
+    case TILE_256x192: return launch_persistent_variant<256, 192, 4, 2, 2, 128>(g, workgroups, s);
+    case TILE_256x128: return launch_persistent_variant<256, 128, 4, 2, 3, 128>(g, workgroups, s);
+    case TILE_128x192: return launch_persistent_variant<128, 192, 4, 2, 3, 128>(g, workgroups, s);
+    case TILE_128x128: return launch_persistent_variant<128, 128, 2, 4, 4, 128>(g, workgroups, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace fp8gemm

@@ -28,6 +28,10 @@ bool tile_supports(const GemmArgs& g);
 const char* tile_variant_name(int variant);
 void tile_variant_dims(int variant, int* bm, int* bn);
 hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, hipStream_t s);
+// Persistent form (ksplit = 1 only): `workgroups` (a multiple of 8) workgroups walk through
+// all tiles, the copies of a tile's first K blocks overlap the previous tile's epilogue.
+bool tile_persistent_supports(const GemmArgs& g, int variant);
+hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups, hipStream_t s);
 hipError_t launch_splitk_reduce(const GemmArgs& g, int ksplit, const float* partial, hipStream_t s);
 
 // tiny-M streaming kernel (decode shapes)

@@ -78,6 +78,12 @@ int fp8_block_gemm_select(int kernel_id);
  * (/root/reference/mn_large.hip:1-8). */
 int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 
+/* The tile kernels have a persistent form (ksplit = 1): 256 workgroups walk through all
+ * tiles and copy a tile's first K blocks while the previous tile is stored.  mode -1 = use it
+ * when there are more tiles than compute units (default), 0 = never, 1 = whenever the shape
+ * allows.  The reference names such a kernel as future work (/root/reference/README.md:29). */
+int fp8_block_gemm_set_persistent(int mode);
+
 /* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
  * 16-byte aligned operands into name[0..cap), e.g. "tile256x256_k1", "skinny_k1", "scalar".
  * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart

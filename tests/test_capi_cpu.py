@@ -59,6 +59,16 @@ def test_select_and_force_config_validate(pkg):
     for kid in (1, 2, 3, 4, 0):
         assert L.fp8_block_gemm_select(kid) == 0
     assert L.fp8_block_gemm_force_config(-1, 0) == 0
+    assert L.fp8_block_gemm_set_persistent(2) == -3
+    assert L.fp8_block_gemm_set_persistent(1) == 0
+    assert pkg.plan(8192, 4608, 7168).endswith("_persistent")
+    assert pkg.plan(2048, 2048, 2048).endswith("_persistent")   # forced: whenever the kernel allows
+    assert pkg.plan(256, 256, 256) == "tile64x64_k1"             # the 64x64 tile has no persistent form
+    assert L.fp8_block_gemm_set_persistent(0) == 0
+    assert not pkg.plan(8192, 4608, 7168).endswith("_persistent")
+    assert L.fp8_block_gemm_set_persistent(-1) == 0
+    assert pkg.plan(8192, 4608, 7168).endswith("_persistent")   # 768 tiles on 256 CUs
+    assert not pkg.plan(2048, 2048, 2048).endswith("_persistent")
 
 
 def test_workspace_contract(pkg):
@@ -75,7 +85,7 @@ def test_dispatcher_plans(pkg):
     pkg.select(pkg.KERNEL_AUTO)
     pkg.force_config(-1, 0)
     assert pkg.plan(8192, 4608, 7168).startswith("tile")
-    assert pkg.plan(8192, 4608, 7168).endswith("_k1")
+    assert "_k1" in pkg.plan(8192, 4608, 7168)
     assert pkg.plan(32, 7168, 2048).startswith("skinny")
     assert pkg.plan(33, 100, 128) == "scalar"            # rows not 16-byte aligned
     ks = int(pkg.plan(2048, 576, 7168).split("_k")[1])

@@ -28,13 +28,15 @@ def _dev(*arrs):
     return [torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in arrs]
 
 
-def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=False):
+def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=False, persistent=-1):
     import torch
     da, db, dsa, dsb = _dev(a, b, sa, sb)
     dc = torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)  # NaN sentinel
-    _say(f"[gpu case] m={m} n={n} k={k} kernel={kernel} variant={variant} ksplit={ksplit} scalar={scalar}")
+    _say(f"[gpu case] m={m} n={n} k={k} kernel={kernel} variant={variant} ksplit={ksplit} scalar={scalar} "
+         f"persistent={persistent}")
     pkg.select(kernel)
     pkg.force_config(variant, ksplit)
+    pkg.set_persistent(persistent)
     try:
         if scalar:
             pkg.gemm_scalar(da, db, dsa, dsb, dc, m, n, k)
@@ -45,6 +47,7 @@ def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=Fals
     finally:
         pkg.select(0)
         pkg.force_config(-1, 0)
+        pkg.set_persistent(-1)
     return dc.cpu().numpy().view(np.uint16), name
 
 
@@ -87,6 +90,23 @@ def test_tile_kernel(pkg, variant, m, n, k):
     got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant)
     assert name.endswith("_k1"), name
     _assert_close(got, ref, name)
+
+
+# persistent form: several tiles per workgroup (more than 256 tiles), ragged edges, K ranges from
+# the shortest the ring allows to many blocks, and a launch with fewer tiles than workgroups
+@pytest.mark.parametrize("variant,m,n,k", [(0, 4096, 3456, 512), (0, 1040, 1232, 256), (0, 4112, 3472, 128),
+                                           (1, 4096, 2176, 384), (1, 4368, 2064, 256),
+                                           (2, 4096, 4096, 384), (2, 2304, 2320, 1024),
+                                           (3, 2064, 4032, 640), (3, 2048, 6528, 256)])
+def test_tile_kernel_persistent(pkg, variant, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, m + 3 * n + k + variant, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant, persistent=1)
+    assert name.endswith("_k1_persistent"), name
+    _assert_close(got, ref, name)
+    plain, name0 = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant, persistent=0)
+    assert name0.endswith("_k1"), name0
+    assert np.array_equal(got, plain), "persistent and plain tile kernels fold the same sums in the same order"
 
 
 @pytest.mark.parametrize("variant,ksplit,m,n,k", [(2, 2, 256, 256, 512), (2, 4, 512, 512, 1024),
