@@ -292,3 +292,25 @@ def test_check_driver_reproduces_the_reference_procedure(pkg):
         out = subprocess.run([exe] + args, capture_output=True, text=True, timeout=120)
         assert out.returncode == 0, out.stdout + out.stderr
         assert "2 matrices are equal" in out.stdout
+
+
+def test_custom_kernel_operator_form(pkg):
+    """torch tensors in the column-major layouts of the challenge harness; fp8 dtype views"""
+    import torch
+    m, n, k = 256, 576, 512
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 321)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    ta = torch.from_numpy(a).cuda().view(torch.float8_e4m3fn).t()        # [m, k], strides (1, m)
+    tb = torch.from_numpy(b).cuda().view(torch.float8_e4m3fn).t()
+    tsa = torch.from_numpy(sa).cuda().t()                                # [m, k/128], strides (1, m)
+    tsb = torch.from_numpy(sb).cuda().t()                                # [ceil(n/128), k/128]
+    c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    _say(f"[gpu case] custom_kernel m={m} n={n} k={k}")
+    out = pkg.custom_kernel((ta, tb, tsa, tsb, c))
+    torch.cuda.synchronize()
+    assert out is c
+    _assert_close(c.view(torch.int16).cpu().numpy().view(np.uint16), ref, "custom_kernel")
+    with pytest.raises(ValueError):
+        pkg.custom_kernel((ta.contiguous(), tb, tsa, tsb, c))            # row-major a is refused
+    with pytest.raises(ValueError):
+        pkg.custom_kernel((ta, tb, tsa, tsb, c.t()))
