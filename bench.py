@@ -44,7 +44,7 @@ CHALLENGE_REF_GEOMEAN_US = 136.0
 # same counter reads for a 1 GiB copy kernel: FETCH_SIZE reads 0.5 of the bytes copied
 # (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).  See profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg4": int((242049 * 2.0 + 75966 * 1.0) * 1024),   # 573 MB: 8 L2s refetch A/B panels
+    "cfg4": int((242100 * 2.0 + 73728 * 1.0) * 1024),   # 571 MB: 8 L2s refetch A/B panels
     "cfg5": int((7462.75 * 2.0 + 448 * 1.0) * 1024),    # 15.7 MB: 1.04 x the algorithmic bytes
 }
 
@@ -246,6 +246,31 @@ def main():
             del x, q, sc
         return out
 
+    def vendor_plain_fp8_gemm_us(steps, warmup):
+        """Context, not a baseline of this metric: torch._scaled_mm (the ROCm library GEMM) on the
+        headline shape with one scale per tensor, i.e. WITHOUT the per-128-K-block fold."""
+        try:
+            xa = torch.randn((m, k), device="cuda").clamp(-3, 3).to(torch.float8_e4m3fn)
+            xb = torch.randn((n, k), device="cuda").clamp(-3, 3).to(torch.float8_e4m3fn)
+            one = torch.tensor(1.0, device="cuda")
+            fn = lambda: torch._scaled_mm(xa, xb.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+            for _ in range(warmup):
+                fn()
+            torch.cuda.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / steps
+            return {"what": "torch._scaled_mm, per-tensor scales (no block-scale fold), same M N K",
+                    "latency_us": round(us, 2), "tflops": round(flops / us * 1e-6, 1),
+                    "frac_fp8_peak": round(flops / us * 1e-6 / PEAK_FP8_TFLOPS, 4)}
+        except Exception as exc:  # library or dtype not available: context only
+            return {"what": "torch._scaled_mm unavailable", "error": repr(exc)[:200]}
+
     def launch_floor_us(reps=200):
         """back-to-back launches of a one-workgroup kernel of this library"""
         x = torch.zeros(256, dtype=torch.float32, device="cuda")
@@ -280,6 +305,7 @@ def main():
         challenge = challenge_report(max(10, args.steps // 2), args.warmup)
     floor_us = launch_floor_us()
     quantisers = None if args.no_shapes else quantiser_report(max(10, args.steps // 2), args.warmup)
+    vendor = None if args.no_shapes else vendor_plain_fp8_gemm_us(max(10, args.steps // 2), args.warmup)
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
               "max_sclk_mhz": max_sclk_mhz(),
@@ -340,6 +366,7 @@ def main():
         "shapes": shapes,
         "challenge": challenge,
         "quantisers": quantisers,
+        "vendor_plain_fp8_gemm": vendor,
         "device": device,
     }
     print(json.dumps(out))

@@ -1,12 +1,16 @@
 // Timing driver: the procedure of /root/reference/sgemm.cu:89-127 (10 launches bracketed by
 // events, first one dropped, mean of the remaining 9 in microseconds), on the full grid
 // (the reference's timed cases launch half of it, sgemm.cu:106).  Inputs are resident on the
-// device before the timed region.  Usage: sgemm M N K [runs [tile_variant [ksplit]]]
-// (tile_variant / ksplit pin the kernel plan as fp8_block_gemm_force_config does)
+// device before the timed region.  Usage: sgemm M N K [runs [tile_variant [ksplit [constant]]]]
+// (tile_variant / ksplit pin the kernel plan as fp8_block_gemm_force_config does, -1 / 0 leave
+// the choice to the dispatcher; constant = 1 fills both operands with the single code 0x38
+// instead of the seed-7 stream: same instructions, no toggling operand bits, i.e. the run
+// time without the power limit that random data hits)
 #include "host_harness.h"
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdlib>
 
 #define CHECK(x)                                                                     \
@@ -29,6 +33,7 @@ int main(int argc, char** argv)
         std::fprintf(stderr, "bad tile_variant / ksplit\n");
         return 2;
     }
+    const bool constant = argc > 7 && std::atoi(argv[7]) != 0;
     const size_t nkb = K / 128, sn = (N + 127) / 128;
 
     // byte patterns straight from the seed-7 stream: any finite e4m3 code
@@ -38,6 +43,10 @@ int main(int argc, char** argv)
         a8[i] = (uint8_t)((int)(fa[i % fa.size()] * 12.f) & 0x77);
     for (size_t i = 0; i < b8.size(); ++i)
         b8[i] = (uint8_t)((int)(fa[(i * 7 + 3) % fa.size()] * 12.f) & 0x77);
+    if (constant) {
+        std::fill(a8.begin(), a8.end(), (uint8_t)0x38);
+        std::fill(b8.begin(), b8.end(), (uint8_t)0x38);
+    }
     std::vector<float> as(nkb * M, 0.01f), bs(nkb * sn, 0.02f);
 
     void *da, *db, *das, *dbs, *dc;
