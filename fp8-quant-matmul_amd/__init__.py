@@ -10,7 +10,7 @@ a failing call raises.
 from .capi import (  # noqa: F401
     Fp8GemmError,
     KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY,
-    DTYPE_BF16, DTYPE_F32, quantize_a_1x128, quantize_b_128x128,
+    DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH, quantize_a_1x128, quantize_b_128x128,
     abi_symbols, build, convert_f32_to_e4m3fn, custom_kernel, error_string, force_config, gemm, gemm_scalar,
     last_kernel, lib, lib_path, plan, release, select, set_persistent, set_workspace, workspace_bytes,
 )

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
 KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5)
-DTYPE_BF16, DTYPE_F32 = 0, 1
+DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH = 0, 1, 2
 
 
 class Fp8GemmError(RuntimeError):

@@ -383,11 +383,14 @@ static int quantize_entry(const void* x, int x_dtype, void* q, float* scale, int
         return FP8GEMM_E_SHAPE;
     if ((long long)rows * k > 0x7FFFFFFFll)
         return FP8GEMM_E_TOOLARGE;
-    if (x_dtype != FP8GEMM_DTYPE_BF16 && x_dtype != FP8GEMM_DTYPE_F32)
+    if (x_dtype != FP8GEMM_DTYPE_BF16 && x_dtype != FP8GEMM_DTYPE_F32 && x_dtype != FP8GEMM_DTYPE_BF16_F32MATH)
         return FP8GEMM_E_DTYPE;
     if (reinterpret_cast<uintptr_t>(x) % 16 != 0)
         return FP8GEMM_E_ALIGN;
-    return (int)launch_quantize(x, x_dtype == FP8GEMM_DTYPE_F32, static_cast<uint8_t*>(q), scale, rows,
+    static_assert(QUANT_SOURCE_BF16 == FP8GEMM_DTYPE_BF16 && QUANT_SOURCE_F32 == FP8GEMM_DTYPE_F32 &&
+                      QUANT_SOURCE_BF16_F32MATH == FP8GEMM_DTYPE_BF16_F32MATH,
+                  "launcher enum mirrors the ABI constants");
+    return (int)launch_quantize(x, static_cast<QuantSource>(x_dtype), static_cast<uint8_t*>(q), scale, rows,
                                 k, block128, static_cast<hipStream_t>(stream));
 }
 

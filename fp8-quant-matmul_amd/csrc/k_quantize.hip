@@ -3,8 +3,14 @@
 //   1 x 128 groups along K per row   (to_float8_rowwise_scale, /root/reference/quantize.py:43-67)
 //   128 x 128 blocks                 (to_float8_block_scale,   /root/reference/quantize.py:16-41)
 //
-// Arithmetic of both, in fp32, with the OCP e4m3fn maximum 448:
-//   scale = 448 / max(amax, 1e-12);  q = fp8_rne(clamp(x * scale, -448, 448));  stored = 1 / scale
+// Arithmetic of both, with the OCP e4m3fn maximum 448:
+//   scale = (1 / max(amax, 1e-12)) * 448;  q = fp8_rne(clamp(x * scale, -448, 448));  stored = 1 / scale
+// (reciprocal first, then the product: that is how torch evaluates `finfo.max / amax`,
+// quantize.py:28,54).  For an fp32 source every step is fp32.  For a bf16 source torch rounds
+// every element-wise result to bf16 (1e-12, the reciprocal, the product with 448, x * scale);
+// BF16MATH reproduces that, so that bytes and scales equal the reference's own outputs for
+// either source type.  A bf16 source can also be quantised with fp32 arithmetic (more
+// accurate, not what quantize.py computes).
 //
 // The source x is row-major [rows][K] (K contiguous), bf16 or fp32.  The outputs are written
 // directly in the GEMM's layouts, which the reference produces with host-side transposes
@@ -52,8 +58,20 @@ __device__ __forceinline__ float clamp_pm448(float v)
     return fminf(fmaxf(v, -448.0f), 448.0f);
 }
 
+template <bool BF16MATH>
+__device__ __forceinline__ float q_round(float v)
+{
+    return BF16MATH ? __uint_as_float(pack_bf16x2(v, 0.0f) << 16) : v;
+}
+
+template <bool BF16MATH>
+__device__ __forceinline__ float q_value(float x, float scale)
+{
+    return clamp_pm448(q_round<BF16MATH>(x * scale));
+}
+
 // BLOCK = false: one scale per row and tile (1 x 128).  BLOCK = true: one per tile (128 x 128).
-template <typename TIn, bool BLOCK>
+template <typename TIn, bool BLOCK, bool BF16MATH>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __restrict__ scale_out,
                 int rows, int K, int vec_store)
@@ -113,12 +131,13 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
         const int r = r0 + 16 * p;
-        const float scale = 448.0f / fmaxf(amax[p], 1e-12f);
+        const float recip = q_round<BF16MATH>(1.0f / fmaxf(amax[p], q_round<BF16MATH>(1e-12f)));
+        const float scale = q_round<BF16MATH>(recip * 448.0f);
         int w0 = 0, w1 = 0;
-        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][0] * scale), clamp_pm448(v[p][1] * scale), w0, false);
-        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][2] * scale), clamp_pm448(v[p][3] * scale), w0, true);
-        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][4] * scale), clamp_pm448(v[p][5] * scale), w1, false);
-        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_pm448(v[p][6] * scale), clamp_pm448(v[p][7] * scale), w1, true);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q_value<BF16MATH>(v[p][0], scale), q_value<BF16MATH>(v[p][1], scale), w0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q_value<BF16MATH>(v[p][2], scale), q_value<BF16MATH>(v[p][3], scale), w0, true);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q_value<BF16MATH>(v[p][4], scale), q_value<BF16MATH>(v[p][5], scale), w1, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q_value<BF16MATH>(v[p][6], scale), q_value<BF16MATH>(v[p][7], scale), w1, true);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             tile[(8 * c + j) * QSTRIDE + r] = (uint8_t)((uint32_t)w0 >> (8 * j));
@@ -154,25 +173,37 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
     }
 }
 
-}  // namespace
-
-hipError_t launch_quantize(const void* x, bool x_is_f32, uint8_t* q, float* scale_out, int rows,
-                           int k, bool block128, hipStream_t s)
+template <typename TIn, bool BF16MATH>
+void launch_quantize_typed(const TIn* x, uint8_t* q, float* scale_out, int rows, int k, bool block128,
+                           hipStream_t s)
 {
     const dim3 grid((rows + QTILE - 1) / QTILE, k / 128);
     const int vec_store = (rows % 16 == 0) && (reinterpret_cast<uintptr_t>(q) % 16 == 0);
-    if (x_is_f32) {
-        const float* xf = static_cast<const float*>(x);
-        if (block128)
-            hipLaunchKernelGGL((quantize_kernel<float, true>), grid, dim3(256), 0, s, xf, q, scale_out, rows, k, vec_store);
-        else
-            hipLaunchKernelGGL((quantize_kernel<float, false>), grid, dim3(256), 0, s, xf, q, scale_out, rows, k, vec_store);
-    } else {
-        const uint16_t* xh = static_cast<const uint16_t*>(x);
-        if (block128)
-            hipLaunchKernelGGL((quantize_kernel<uint16_t, true>), grid, dim3(256), 0, s, xh, q, scale_out, rows, k, vec_store);
-        else
-            hipLaunchKernelGGL((quantize_kernel<uint16_t, false>), grid, dim3(256), 0, s, xh, q, scale_out, rows, k, vec_store);
+    if (block128)
+        hipLaunchKernelGGL((quantize_kernel<TIn, true, BF16MATH>), grid, dim3(256), 0, s, x, q, scale_out, rows,
+                           k, vec_store);
+    else
+        hipLaunchKernelGGL((quantize_kernel<TIn, false, BF16MATH>), grid, dim3(256), 0, s, x, q, scale_out, rows,
+                           k, vec_store);
+}
+
+}  // namespace
+
+hipError_t launch_quantize(const void* x, QuantSource source, uint8_t* q, float* scale_out, int rows,
+                           int k, bool block128, hipStream_t s)
+{
+    switch (source) {
+    case QUANT_SOURCE_BF16:
+        launch_quantize_typed<uint16_t, true>(static_cast<const uint16_t*>(x), q, scale_out, rows, k, block128, s);
+        break;
+    case QUANT_SOURCE_F32:
+        launch_quantize_typed<float, false>(static_cast<const float*>(x), q, scale_out, rows, k, block128, s);
+        break;
+    case QUANT_SOURCE_BF16_F32MATH:
+        launch_quantize_typed<uint16_t, false>(static_cast<const uint16_t*>(x), q, scale_out, rows, k, block128, s);
+        break;
+    default:
+        return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }

@@ -44,7 +44,9 @@ hipError_t launch_convert(const float* in, uint8_t* out, size_t count, hipStream
 
 // 1 x 128 (block128 = false) or 128 x 128 quantiser of a row-major [rows][k] matrix into the
 // GEMM's column-major fp8 layout and scale layout (quantize.py:16-67)
-hipError_t launch_quantize(const void* x, bool x_is_f32, uint8_t* q, float* scale_out, int rows,
+// source: element type of x and the arithmetic (values of FP8GEMM_DTYPE_*)
+enum QuantSource { QUANT_SOURCE_BF16 = 0, QUANT_SOURCE_F32 = 1, QUANT_SOURCE_BF16_F32MATH = 2 };
+hipError_t launch_quantize(const void* x, QuantSource source, uint8_t* q, float* scale_out, int rows,
                            int k, bool block128, hipStream_t s);
 
 }  // namespace fp8gemm

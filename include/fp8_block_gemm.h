@@ -37,9 +37,14 @@ extern "C" {
 #define FP8GEMM_E_DTYPE (-6)     /* unknown FP8GEMM_DTYPE_* value */
 #define FP8GEMM_E_ALIGN (-7)     /* a source pointer is not 16-byte aligned */
 
-/* Element types of a quantiser's source matrix. */
+/* Element type of a quantiser's source matrix, and with it the arithmetic: quantize.py computes
+ * in the tensor's own dtype, i.e. torch rounds every element-wise result to bf16 for a bf16
+ * tensor.  BF16 and F32 reproduce the reference's outputs bit for bit for that source type;
+ * BF16_F32MATH reads bf16 but keeps fp32 intermediates (more accurate, not what quantize.py
+ * computes). */
 #define FP8GEMM_DTYPE_BF16 0
 #define FP8GEMM_DTYPE_F32 1
+#define FP8GEMM_DTYPE_BF16_F32MATH 2
 
 /* Kernel ids for fp8_block_gemm_select (the run-time counterpart of the reference's
  * compile-time OPTION / #include swap, mn_large.hip:9, check.cu:13). */
@@ -111,8 +116,9 @@ int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* st
 
 /* Quantise activations for the GEMM's `a` operand: x is [m][k] row-major (k contiguous),
  * bf16 or fp32 (x_dtype = FP8GEMM_DTYPE_*), 16-byte aligned.  Per row and 128-wide K group:
- * scale = 448 / max(amax, 1e-12), a = fp8_rne(clamp(x * scale, +-448)) written at m + k*M,
- * a_scale = 1 / scale written at m + kb*M, all in fp32 arithmetic.  Replaces
+ * scale = (1 / max(amax, 1e-12)) * 448 (torch's evaluation order of finfo.max / amax),
+ * a = fp8_rne(clamp(x * scale, +-448)) written at m + k*M, a_scale = 1 / scale written at
+ * m + kb*M.  Replaces
  * to_float8_rowwise_scale (/root/reference/quantize.py:43-67, with the e4m3fn maximum 448
  * instead of fnuz's 240) together with the host-side transposes that bring its outputs into
  * the kernel's layouts (row_to_col_major, /root/reference/check.cu:164-167). */

@@ -65,9 +65,9 @@ def lib():
     L.oracle_gen_normal_bf16.argtypes = [f32p, C.c_size_t, C.c_size_t, C.c_uint64, C.c_double,
                                          C.c_double]
     L.oracle_quantize_a_1x128.restype = None
-    L.oracle_quantize_a_1x128.argtypes = [f32p, u8p, f32p, C.c_int, C.c_int]
+    L.oracle_quantize_a_1x128.argtypes = [f32p, u8p, f32p, C.c_int, C.c_int, C.c_int]
     L.oracle_quantize_b_128x128.restype = None
-    L.oracle_quantize_b_128x128.argtypes = [f32p, u8p, f32p, C.c_int, C.c_int]
+    L.oracle_quantize_b_128x128.argtypes = [f32p, u8p, f32p, C.c_int, C.c_int, C.c_int]
     L.oracle_make_inputs.restype = None
     L.oracle_make_inputs.argtypes = [u8p, u8p, f32p, f32p, C.c_int, C.c_int, C.c_int, C.c_uint64,
                                      C.c_double, C.c_double]
@@ -173,25 +173,26 @@ def gen_normal_bf16(rows, cols, seed, outlier_pct=0.0, outlier_mul=1.0):
     return out
 
 
-def quantize_a_1x128(x):
-    """x: [M, K] fp32 row-major -> (bytes laid out m + k*M as array [K, M], a_scale [K/128, M])."""
+def quantize_a_1x128(x, bf16_arith=False):
+    """x: [M, K] fp32 row-major -> (bytes laid out m + k*M as array [K, M], a_scale [K/128, M]).
+    bf16_arith: round every intermediate to bf16, as torch does when quantize.py gets a bf16 tensor."""
     x = np.ascontiguousarray(x, np.float32)
     m, k = x.shape
     assert k % 128 == 0
     q = np.empty((k, m), np.uint8)
     s = np.empty((k // 128, m), np.float32)
-    lib().oracle_quantize_a_1x128(_p(x), _p(q), _p(s), m, k)
+    lib().oracle_quantize_a_1x128(_p(x), _p(q), _p(s), m, k, int(bool(bf16_arith)))
     return q, s
 
 
-def quantize_b_128x128(x):
+def quantize_b_128x128(x, bf16_arith=False):
     """x: [N, K] fp32 row-major -> (bytes n + k*N as array [K, N], b_scale [K/128, ceil(N/128)])."""
     x = np.ascontiguousarray(x, np.float32)
     n, k = x.shape
     assert k % 128 == 0
     q = np.empty((k, n), np.uint8)
     s = np.empty((k // 128, (n + 127) // 128), np.float32)
-    lib().oracle_quantize_b_128x128(_p(x), _p(q), _p(s), n, k)
+    lib().oracle_quantize_b_128x128(_p(x), _p(q), _p(s), n, k, int(bool(bf16_arith)))
     return q, s
 
 

@@ -12,9 +12,9 @@
  *     "result += block * as * bs" evaluated left to right, final cast to bf16)
  *   - /root/reference/utils.h:65-76   (gemmCPU: the i / j / t host loop nest)
  *   - /root/reference/check.cu:17-22  (convert_float_to_fp8: fp32 -> fp8, saturating, RNE)
- *   - /root/reference/quantize.py:16-67 (1x128 and 128x128 quantisers; scale = max/amax,
- *     returned inverse scale = 1/scale), with FP8 max = 448 (OCP e4m3fn) instead of the
- *     MI300 fnuz flavour.
+ *   - /root/reference/quantize.py:16-67 (1x128 and 128x128 quantisers; scale = max/amax as
+ *     torch evaluates it, returned inverse scale = 1/scale), with FP8 max = 448 (OCP e4m3fn)
+ *     instead of the MI300 fnuz flavour.
  *
  * Layouts (check.cu:42-48):  a byte at m + k*M, b byte at n + k*N, a_scale at m + kb*M,
  * b_scale at nb + kb*ceil(N/128), c at m*N + n.
@@ -26,8 +26,9 @@
  *   ref_gemm     - exact int64 fixed-point block sums -> fp64 (oracle_ref_gemm_f64),
  *                  numpy matmul for unit scales, one-hot index pins, Fraction brute force,
  *                  the reference's own gemmCPU/genMat built from its header where available
- *   quantisers   - closed-form invariants (max code 448 per group, half-ulp error bound,
- *                  zero group), layout pins
+ *   quantisers   - the reference's own outputs for fp32 and bf16 sources, bit for bit
+ *                  (tests/golden/quantize_reference.npz), closed-form invariants (max code 448
+ *                  per group, half-ulp error bound, zero group), layout pins
  * ref_gemm_rows (the n-vectorised loop order) is pinned bit-for-bit to ref_gemm_naive.
  */
 #include <math.h>
@@ -331,12 +332,41 @@ void oracle_gen_normal_bf16(float *out, size_t rows, size_t cols, uint64_t seed,
         }
 }
 
-/* quantize.py:43-67 (to_float8_rowwise_scale) with FP8 max 448, fp32 arithmetic:
- * per row and 128-wide K group  scale = 448 / max(amax, 1e-12),
- * q = fp8(clamp(x * scale, +-448)), stored inverse scale = 1 / scale.
+/* The quantisers of quantize.py with FP8 max 448 (torch.float8_e4m3fn).  Per scale group:
+ *     amax' = max(amax, 1e-12)
+ *     scale = (1 / amax') * 448        two roundings: torch evaluates `finfo.max / tensor`
+ *                                      (quantize.py:28,54) as tensor.reciprocal() * finfo.max
+ *     q     = fp8_rne(clamp(x * scale, +-448))
+ *     stored inverse scale = 1 / scale (quantize.py:39,65: scale.float().reciprocal())
+ * bf16_arith = 0: every step in fp32 (what torch does for an fp32 tensor).
+ * bf16_arith = 1: what torch does for a bf16 tensor, whose element-wise results are rounded to
+ *     bf16 after every operation: 1e-12, the reciprocal, the product with 448 and x * scale are
+ *     each rounded to bf16; the stored inverse scale is the fp32 reciprocal of the bf16 scale.
+ * Both forms reproduce the reference's own outputs bit for bit
+ * (tests/golden/quantize_reference.npz, written by importing quantize.py). */
+static inline float q_round(float v, int bf16_arith)
+{
+    return bf16_arith ? oracle_bf16_to_f32(oracle_f32_to_bf16(v)) : v;
+}
+
+static inline float q_scale(float amax, int bf16_arith)
+{
+    float floor_ = q_round(1e-12f, bf16_arith);
+    float r = q_round(1.0f / fmaxf(amax, floor_), bf16_arith);
+    return q_round(r * 448.0f, bf16_arith);
+}
+
+static inline uint8_t q_code(float x, float scale, int bf16_arith)
+{
+    float v = q_round(x * scale, bf16_arith);
+    v = fminf(fmaxf(v, -448.0f), 448.0f);
+    return oracle_f32_to_e4m3fn(v);
+}
+
+/* quantize.py:43-67 (to_float8_rowwise_scale): one scale per row and 128-wide K group.
  * x is M x K row-major.  Outputs are written in the kernel's layouts (the transposes the
  * reference leaves to its host code, check.cu:164-167): q at m + k*M, a_scale at m + kb*M. */
-void oracle_quantize_a_1x128(const float *x, uint8_t *q, float *a_scale, int m, int k)
+void oracle_quantize_a_1x128(const float *x, uint8_t *q, float *a_scale, int m, int k, int bf16_arith)
 {
     int nkb = k / KBLK;
 #pragma omp parallel for schedule(static)
@@ -346,21 +376,18 @@ void oracle_quantize_a_1x128(const float *x, uint8_t *q, float *a_scale, int m, 
             float amax = 0.0f;
             for (int t = 0; t < KBLK; ++t)
                 amax = fmaxf(amax, fabsf(g[t]));
-            float scale = 448.0f / fmaxf(amax, 1e-12f);
-            for (int t = 0; t < KBLK; ++t) {
-                float v = g[t] * scale;
-                v = fminf(fmaxf(v, -448.0f), 448.0f);
-                q[(size_t)i + (size_t)(kb * KBLK + t) * m] = oracle_f32_to_e4m3fn(v);
-            }
+            float scale = q_scale(amax, bf16_arith);
+            for (int t = 0; t < KBLK; ++t)
+                q[(size_t)i + (size_t)(kb * KBLK + t) * m] = q_code(g[t], scale, bf16_arith);
             a_scale[(size_t)i + (size_t)kb * m] = 1.0f / scale;
         }
 }
 
 /* quantize.py:16-41 (to_float8_block_scale), same arithmetic per 128 x 128 block.
  * x is N x K row-major.  N need not be a multiple of 128: the last block's amax is taken
- * over the rows that exist (equivalent to zero padding).  Outputs: q at n + k*N,
- * b_scale at nb + kb*ceil(N/128). */
-void oracle_quantize_b_128x128(const float *x, uint8_t *q, float *b_scale, int n, int k)
+ * over the rows that exist (equivalent to zero padding; quantize.py:23-26 drops such rows).
+ * Outputs: q at n + k*N, b_scale at nb + kb*ceil(N/128). */
+void oracle_quantize_b_128x128(const float *x, uint8_t *q, float *b_scale, int n, int k, int bf16_arith)
 {
     int nkb = k / KBLK, sn = (n + KBLK - 1) / KBLK;
 #pragma omp parallel for schedule(static) collapse(2)
@@ -371,13 +398,11 @@ void oracle_quantize_b_128x128(const float *x, uint8_t *q, float *b_scale, int n
             for (int r = nb * KBLK; r < r1; ++r)
                 for (int t = 0; t < KBLK; ++t)
                     amax = fmaxf(amax, fabsf(x[(size_t)r * k + (size_t)kb * KBLK + t]));
-            float scale = 448.0f / fmaxf(amax, 1e-12f);
+            float scale = q_scale(amax, bf16_arith);
             for (int r = nb * KBLK; r < r1; ++r)
-                for (int t = 0; t < KBLK; ++t) {
-                    float v = x[(size_t)r * k + (size_t)kb * KBLK + t] * scale;
-                    v = fminf(fmaxf(v, -448.0f), 448.0f);
-                    q[(size_t)r + (size_t)(kb * KBLK + t) * n] = oracle_f32_to_e4m3fn(v);
-                }
+                for (int t = 0; t < KBLK; ++t)
+                    q[(size_t)r + (size_t)(kb * KBLK + t) * n] =
+                        q_code(x[(size_t)r * k + (size_t)kb * KBLK + t], scale, bf16_arith);
             b_scale[(size_t)nb + (size_t)kb * sn] = 1.0f / scale;
         }
 }
@@ -391,8 +416,8 @@ void oracle_make_inputs(uint8_t *a, uint8_t *b, float *a_scale, float *b_scale, 
     float *xb = (float *)malloc((size_t)n * k * sizeof(float));
     oracle_gen_normal_bf16(xa, (size_t)m, (size_t)k, seed * 2 + 1, a_outlier_pct, a_outlier_mul);
     oracle_gen_normal_bf16(xb, (size_t)n, (size_t)k, seed * 2 + 2, 0.0, 1.0);
-    oracle_quantize_a_1x128(xa, a, a_scale, m, k);
-    oracle_quantize_b_128x128(xb, b, b_scale, n, k);
+    oracle_quantize_a_1x128(xa, a, a_scale, m, k, 0);
+    oracle_quantize_b_128x128(xb, b, b_scale, n, k, 0);
     free(xa);
     free(xb);
 }

@@ -1,8 +1,10 @@
 """GPU parity of the device-side quantisers against the CPU oracle, through the C ABI.
 
 Bar: bit-exact.  fp8 bytes and fp32 scales are the results of a handful of IEEE fp32
-operations (max, one division, one multiplication, a clamp, one rounding to e4m3fn, one
-division) that are the same on both sides, so every byte and every scale bit must agree.
+operations (max, a reciprocal, two multiplications, a clamp, one rounding to e4m3fn, a
+reciprocal; with a bf16 source a rounding to bf16 after each) that are the same on both sides,
+so every byte and every scale bit must agree -- with the oracle, and with the reference's own
+quantize.py outputs held in tests/golden/quantize_reference.npz.
 """
 import sys
 
@@ -29,7 +31,7 @@ def _bf16_bits(x):
 def _quantize_gpu(pkg, x, which, dtype):
     import torch
     rows, k = x.shape
-    src = _bf16_bits(x).view(np.int16) if dtype == pkg.DTYPE_BF16 else np.ascontiguousarray(x, np.float32)
+    src = np.ascontiguousarray(x, np.float32) if dtype == pkg.DTYPE_F32 else _bf16_bits(x).view(np.int16)
     dx = torch.from_numpy(src).cuda()
     dq = torch.full((k, rows), 0x7F, dtype=torch.uint8, device="cuda")          # NaN code sentinel
     ncol = rows if which == "a" else (rows + 127) // 128
@@ -43,7 +45,8 @@ def _quantize_gpu(pkg, x, which, dtype):
 
 def _check(pkg, x, which, dtype):
     q, s = _quantize_gpu(pkg, x, which, dtype)
-    rq, rs = (oracle.quantize_a_1x128 if which == "a" else oracle.quantize_b_128x128)(x)
+    rq, rs = (oracle.quantize_a_1x128 if which == "a" else oracle.quantize_b_128x128)(
+        x, bf16_arith=(dtype == pkg.DTYPE_BF16))
     assert np.array_equal(s.view(np.uint32), rs.view(np.uint32)), (which, x.shape, "scales differ")
     bad = np.argwhere(q != rq)
     assert bad.size == 0, (which, x.shape, bad[:4], q[tuple(bad[0])], rq[tuple(bad[0])])
@@ -59,12 +62,32 @@ SHAPES_B = [(512, 2048), (576, 7168), (7168, 2048), (128, 128), (64, 128), (1, 2
 def test_quantize_a_bf16_matches_oracle(pkg, rows, k):
     x = oracle.gen_normal_bf16(rows, k, 31 + rows + k, 1.0, 50.0)
     _check(pkg, x, "a", pkg.DTYPE_BF16)
+    _check(pkg, x, "a", pkg.DTYPE_BF16_F32MATH)
 
 
 @pytest.mark.parametrize("rows,k", SHAPES_B)
 def test_quantize_b_bf16_matches_oracle(pkg, rows, k):
     x = oracle.gen_normal_bf16(rows, k, 57 + rows + k)
     _check(pkg, x, "b", pkg.DTYPE_BF16)
+    _check(pkg, x, "b", pkg.DTYPE_BF16_F32MATH)
+
+
+@pytest.mark.parametrize("tag", ["f32", "bf16"])
+def test_quantize_reproduces_the_reference_outputs(pkg, tag):
+    """the reference's own quantize.py outputs (tests/golden/quantize_reference.npz), bit for bit"""
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "quantize_reference.npz"))
+    x = d["x_f32"]
+    if tag == "bf16":
+        u = x.view(np.uint32)
+        x = ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32).view(np.float32)
+    dtype = pkg.DTYPE_F32 if tag == "f32" else pkg.DTYPE_BF16
+    q, s = _quantize_gpu(pkg, x, "a", dtype)
+    assert np.array_equal(q.T, d[f"rowwise_{tag}_q"])
+    assert np.array_equal(s.T.view(np.uint32), d[f"rowwise_{tag}_s"].view(np.uint32))
+    q, s = _quantize_gpu(pkg, x, "b", dtype)
+    assert np.array_equal(q.T, d[f"block_{tag}_q"])
+    assert np.array_equal(s.T.view(np.uint32), d[f"block_{tag}_s"].view(np.uint32))
 
 
 @pytest.mark.parametrize("which,rows,k", [("a", 256, 512), ("a", 48, 256), ("b", 256, 512),
@@ -88,9 +111,11 @@ def test_quantize_special_groups(pkg):
     x[11, 385] = np.float32(-3.0)
     for which in ("a", "b"):
         _check(pkg, x, which, pkg.DTYPE_BF16)
+        _check(pkg, x, which, pkg.DTYPE_BF16_F32MATH)
         _check(pkg, x * np.float32(1.0 + 2.0 ** -20), which, pkg.DTYPE_F32)
-    q, s = _quantize_gpu(pkg, x, "a", pkg.DTYPE_BF16)
-    assert (q[128:256, 3] == 0).all() and s[1, 3] == np.float32(1.0) / (np.float32(448.0) / np.float32(1e-12))
+    q, s = _quantize_gpu(pkg, x, "a", pkg.DTYPE_BF16_F32MATH)
+    assert (q[128:256, 3] == 0).all()
+    assert s[1, 3] == np.float32(1.0) / ((np.float32(1.0) / np.float32(1e-12)) * np.float32(448.0))
     assert (q[384:512, 11] & 0x7F == 0x7E).all()          # +-448 everywhere
 
 
@@ -115,8 +140,9 @@ def test_gemm_on_device_quantised_inputs_equals_gemm_on_oracle_inputs(pkg):
     pkg.quantize_b_128x128(dxb, db, dsb, n, k, pkg.DTYPE_BF16, st)
     pkg.gemm(da, db, dsa, dsb, dc, m, n, k, st)
     torch.cuda.synchronize()
-    a, sa = oracle.quantize_a_1x128(xa)
-    b, sb = oracle.quantize_b_128x128(xb)
+    a, sa = oracle.quantize_a_1x128(xa, bf16_arith=True)
+    b, sb = oracle.quantize_b_128x128(xb, bf16_arith=True)
+    assert np.array_equal(da.cpu().numpy(), a) and np.array_equal(db.cpu().numpy(), b)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
     r = oracle.compare_bf16(dc.cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)
     assert r["bad"] == 0, r

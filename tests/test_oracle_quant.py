@@ -1,8 +1,14 @@
 """Pins of the oracle's input producers (quantisers and the seeded generator).
 
-quantize.py of the reference is read, not run: the checks are the closed-form invariants its
-arithmetic implies (quantize.py:26-41, 53-67) with FP8 max = 448.
+Two kinds of pins: the closed-form invariants that quantize.py's arithmetic implies
+(quantize.py:26-41, 53-67) with FP8 max = 448, and the reference's own outputs
+(tests/golden/quantize_reference.npz, written by tests/golden/make_quantize_golden.py, which
+imports quantize.py where the reference checkout exists), which fix what the invariants leave
+open: the evaluation order and rounding of the scale and of the scaled values, for fp32 and for
+bf16 sources.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -44,12 +50,41 @@ def test_b_quantiser_invariants_partial_block():
             assert np.all(np.abs(d.T * s[kb, nb] - blk) <= np.abs(blk) * 2.0 ** -4 * 1.001 + s[kb, nb] * 2.0 ** -10 * 1.001)
 
 
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "quantize_reference.npz")
+
+
+def _bf16_round(x):
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32).view(np.float32)
+
+
+@pytest.mark.parametrize("tag", ["f32", "bf16"])
+def test_quantisers_reproduce_the_reference_outputs_bit_for_bit(tag):
+    """quantize.py's outputs are row-major [rows, K] bytes and [rows(/128), K/128] inverse
+    scales; the oracle writes the kernel layouts, i.e. their transposes (check.cu:164-167)."""
+    d = np.load(GOLDEN)
+    x = d["x_f32"] if tag == "f32" else _bf16_round(d["x_f32"])
+    q, s = oracle.quantize_a_1x128(x, bf16_arith=(tag == "bf16"))
+    assert np.array_equal(q.T, d[f"rowwise_{tag}_q"])
+    assert np.array_equal(s.T.view(np.uint32), d[f"rowwise_{tag}_s"].view(np.uint32))
+    q, s = oracle.quantize_b_128x128(x, bf16_arith=(tag == "bf16"))
+    assert np.array_equal(q.T, d[f"block_{tag}_q"])
+    assert np.array_equal(s.T.view(np.uint32), d[f"block_{tag}_s"].view(np.uint32))
+
+
+def test_bf16_source_with_fp32_arithmetic_is_not_the_reference():
+    """the two arithmetics differ on a few percent of the bytes: the vectors tell them apart"""
+    d = np.load(GOLDEN)
+    q, _ = oracle.quantize_a_1x128(_bf16_round(d["x_f32"]), bf16_arith=False)
+    assert 0.001 < (q.T != d["rowwise_bf16_q"]).mean() < 0.2
+
+
 def test_zero_group_gets_tiny_scale_and_zero_codes():
     x = np.zeros((2, 128), np.float32)
     x[1, 3] = 1.0
     q, s = oracle.quantize_a_1x128(x)
     assert not q[:, 0].any()
-    assert s[0, 0] == np.float32(1.0) / (np.float32(448.0) / np.float32(1e-12))
+    assert s[0, 0] == np.float32(1.0) / ((np.float32(1.0) / np.float32(1e-12)) * np.float32(448.0))
     assert oracle.e4m3fn_decode(q[3:4, 1:2])[0, 0] == 448.0
 
 
