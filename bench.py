@@ -11,9 +11,13 @@ and listed under "shapes" with the geomean latency.  "challenge" holds the 18 sh
 reference's own results table (/root/reference/README.md:15-25, measured there on an MI300X)
 with this library's latency on each and the geomean of the 18.  One JSON line is printed.
 
-Timing: W untimed warm-up steps, then exactly K steps between two device synchronisations
-(wall clock -> ms_per_step, value) and between two HIP events recorded on the launch stream
-(-> roofline.achieved: algorithmic flops or bytes of one launch / average launch duration).
+Timing: W untimed warm-up steps -- and as many more as it takes to keep the device under this
+load for SETTLE_MS: after any idle gap, however short, the part needs about 30 ms of continuous
+work to reach its steady clock (the first launches of the headline shape take 340 us, the
+hundredth 240 us, and it stays there) --, then exactly K steps between two device
+synchronisations (wall clock -> ms_per_step, value) and between two HIP events recorded on the
+launch stream (-> roofline.achieved: algorithmic flops or bytes of one launch / average launch
+duration).
 cpu_baseline times the CPU oracle (the restatement of the reference's arithmetic) on a
 bounded row slice of the same workload with all host threads.
 """
@@ -29,6 +33,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5033.0   # 256 CU x 2.4 GHz x 8192 flop/CU/clk (dense, v_mfma_f32_16x16x128_f8f6f4)
 PEAK_HBM_GBS = 8000.0
+SETTLE_MS = 80.0            # continuous load before a timed region (steady device clock)
 HBM_BOUND = {"cfg5"}
 COLD_TOO = {"cfg1", "cfg3", "cfg5"}   # latency-bound shapes: also timed behind a cache flush
 
@@ -128,10 +133,27 @@ def main():
         r = oracle.compare_bf16(got, refh, 1e-2, 1e-3)
         return {"points": npts, "max_err": r["max_err"], "bound": r["bound"], "pass": r["bad"] == 0}
 
-    def timed(dev, dc, shape, steps, warmup):
-        for _ in range(warmup):
-            step(dev, dc, shape)
-        torch.cuda.synchronize()
+    def settle(fn, warmup):
+        """warm-up: at least `warmup` calls of fn, and at least SETTLE_MS of continuous load"""
+        t0 = time.perf_counter()
+        done, batch, per_call_ms = 0, max(warmup, 10), 0.0
+        while done < warmup or (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+            tb = time.perf_counter()
+            for _ in range(batch):
+                fn()
+            done += batch
+            torch.cuda.synchronize()
+            per_call_ms = (time.perf_counter() - tb) * 1e3 / batch
+            if per_call_ms * batch < 5.0:
+                batch *= 2   # short kernels: fewer synchronisation gaps in the load
+        return per_call_ms
+
+    def timed(dev, dc, shape, steps, warmup, exact=False):
+        """(wall ms, event ms) per step over `steps` steps; unless `exact`, short kernels get
+        more steps, so that the timed region lasts 5 ms and its start-up gap does not count"""
+        per_call_ms = settle(lambda: step(dev, dc, shape), warmup)
+        if not exact and per_call_ms > 0:
+            steps = max(steps, int(5.0 / per_call_ms))
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
@@ -172,12 +194,12 @@ def main():
         ts.sort()
         return ts[len(ts) // 2]
 
-    def shape_report(name, steps, warmup):
+    def shape_report(name, steps, warmup, exact=False):
         shape, host, dev, dc = prepare(name)
         step(dev, dc, shape)
         torch.cuda.synchronize()
         par = parity(host, dc, shape)
-        wall_ms, ev_ms = timed(dev, dc, shape, steps, warmup)
+        wall_ms, ev_ms = timed(dev, dc, shape, steps, warmup, exact)
         flops, byts = algorithmic_work(*shape)
         us = ev_ms * 1e3
         rep = {
@@ -227,9 +249,7 @@ def main():
             ncol = rows if which == "a_1x128" else (rows + 127) // 128
             sc = torch.empty((k // 128, ncol), dtype=torch.float32, device="cuda")
             fn = pkg.quantize_a_1x128 if which == "a_1x128" else pkg.quantize_b_128x128
-            for _ in range(warmup):
-                fn(x, q, sc, rows, k, pkg.DTYPE_BF16, sptr)
-            torch.cuda.synchronize()
+            settle(lambda: fn(x, q, sc, rows, k, pkg.DTYPE_BF16, sptr), warmup)
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             e0.record(stream)
@@ -254,9 +274,7 @@ def main():
             xb = torch.randn((n, k), device="cuda").clamp(-3, 3).to(torch.float8_e4m3fn)
             one = torch.tensor(1.0, device="cuda")
             fn = lambda: torch._scaled_mm(xa, xb.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
-            for _ in range(warmup):
-                fn()
-            torch.cuda.synchronize()
+            settle(fn, warmup)
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             e0.record(stream)
@@ -287,7 +305,7 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / reps
 
-    main_rep, (shape, host, wall_ms, ev_ms) = shape_report(args.workload, args.steps, args.warmup)
+    main_rep, (shape, host, wall_ms, ev_ms) = shape_report(args.workload, args.steps, args.warmup, exact=True)
     m, n, k = shape
     flops, byts = algorithmic_work(m, n, k)
 
@@ -304,7 +322,7 @@ def main():
     if not args.no_challenge:
         challenge = challenge_report(max(10, args.steps // 2), args.warmup)
     floor_us = launch_floor_us()
-    quantisers = None if args.no_shapes else quantiser_report(max(10, args.steps // 2), args.warmup)
+    quantisers = None if args.no_shapes else quantiser_report(max(100, args.steps), args.warmup)
     vendor = None if args.no_shapes else vendor_plain_fp8_gemm_us(max(10, args.steps // 2), args.warmup)
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,

@@ -231,12 +231,6 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
             fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
             fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
         }
-        float s[MI], s_hi[MI];
-#pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            s[i] = sa[i] * sb_lo;
-            s_hi[i] = sa[i] * sb_hi;
-        }
 
         // the wave's NCOPY copy instructions of block kb+NS-1 ride on the first MFMAs
         constexpr int N_MFMA = MI * NJ * 2;
@@ -271,7 +265,8 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
             }
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
-                const float sc = patch_hi[j] ? s_hi[i] : s[i];
+                // wave-uniform choice of the b_scale value (a scalar select), one product per patch
+                const float sc = sa[i] * (patch_hi[j] ? sb_hi : sb_lo);
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);

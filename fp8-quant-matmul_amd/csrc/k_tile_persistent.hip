@@ -220,12 +220,6 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
                 fa[i][0] = read_frag(addr_a[i] + so, 0, RSA);
                 fa[i][1] = read_frag(addr_a[i] + so, 1, RSA);
             }
-            float s[MI], s_hi[MI];
-#pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                s[i] = sa[i] * sb_lo;
-                s_hi[i] = sa[i] * sb_hi;
-            }
             constexpr int N_MFMA = MI * NJ * 2;
             constexpr int PER_MFMA = (NCOPY + N_MFMA - 1) / N_MFMA;
             int cq = 0;
@@ -257,7 +251,8 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
                 }
 #pragma unroll
                 for (int i = 0; i < MI; ++i) {
-                    const float sc = patch_hi[jj] ? s_hi[i] : s[i];
+                    // wave-uniform choice of the b_scale value (a scalar select), one product per patch
+                    const float sc = sa[i] * (patch_hi[jj] ? sb_hi : sb_lo);
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
                         acc[i][jj][r] = fmaf(sc, blk[i][r], acc[i][jj][r]);
