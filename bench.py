@@ -15,9 +15,10 @@ Timing: W untimed warm-up steps -- and as many more as it takes to keep the devi
 load for SETTLE_MS: after any idle gap, however short, the part needs about 30 ms of continuous
 work to reach its steady clock (the first launches of the headline shape take 340 us, the
 hundredth 240 us, and it stays there) --, then exactly K steps between two device
-synchronisations (wall clock -> ms_per_step, value) and between two HIP events recorded on the
-launch stream (-> roofline.achieved: algorithmic flops or bytes of one launch / average launch
-duration).
+synchronisations (wall clock -> ms_per_step, value), then a region of at least K steps and at
+least 5 ms between two HIP events recorded on the launch stream, entered without an idle gap
+(-> roofline.achieved: algorithmic flops or bytes of one launch / average launch duration; the
+per-shape latencies are this figure).
 cpu_baseline times the CPU oracle (the restatement of the reference's arithmetic) on a
 bounded row slice of the same workload with all host threads.
 """
@@ -149,21 +150,35 @@ def main():
         return per_call_ms
 
     def timed(dev, dc, shape, steps, warmup, exact=False):
-        """(wall ms, event ms) per step over `steps` steps; unless `exact`, short kernels get
-        more steps, so that the timed region lasts 5 ms and its start-up gap does not count"""
-        per_call_ms = settle(lambda: step(dev, dc, shape), warmup)
-        if not exact and per_call_ms > 0:
-            steps = max(steps, int(5.0 / per_call_ms))
+        """(wall ms, event ms) per step.  The event figure comes from a region of at least
+        `steps` steps and at least 5 ms, entered straight from the warm-up load without a
+        host synchronisation: after any idle gap the first launches are slow, which a region of
+        thirty 5-us kernels would mostly measure.  With `exact`, the wall figure is taken
+        over exactly `steps` steps between two device synchronisations."""
+        run = lambda: step(dev, dc, shape)
+        per_call_ms = settle(run, warmup)
+        wall_ms = None
+        if exact:
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                run()
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        ev_steps = max(steps, int(5.0 / per_call_ms)) if per_call_ms > 0 else steps
+        bridge = max(1, min(ev_steps, int(0.5 / per_call_ms))) if per_call_ms > 0 else 1
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        for _ in range(bridge):   # untimed: the queue is busy when the first event is reached
+            run()
         e0.record(stream)
-        for _ in range(steps):
-            step(dev, dc, shape)
+        for _ in range(ev_steps):
+            run()
         e1.record(stream)
         torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3
-        return wall_ms / steps, e0.elapsed_time(e1) / steps
+        if wall_ms is None:
+            wall_ms = (time.perf_counter() - t0) * 1e3 / (bridge + ev_steps)
+        return wall_ms, e0.elapsed_time(e1) / ev_steps
 
     def launch_stats_us(dev, dc, shape, reps=20):
         """median and minimum of single launches, each between its own pair of events"""
