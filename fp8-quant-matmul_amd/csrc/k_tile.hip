@@ -17,7 +17,10 @@
 //     a_scale[kb][m] * b_scale[kb][n/128] by one FMA per element (mn_large.hip:100-106,
 //     mn_small.hip:85-88 do the same with a second full-size accumulator).
 //   * The MFMA computes the transposed patch (rows = n, columns = m) as mn_small.hip does,
-//     so that a lane owns one m (one a_scale value) and runs of 4 consecutive n (8-byte stores).
+//     so that a lane owns one m (one a_scale value) and runs of 4 consecutive n.
+//   * The finished tile goes through the idle LDS ring (row-major, padded rows) and leaves as
+//     16 bytes per lane along whole tile rows; straight from the accumulators a store
+//     instruction would write 8-byte pieces of 32 different rows.
 //   * a_scale values of the tile travel through LDS with the stage (one extra 1 KiB copy), so
 //     the K loop holds no compiler-visible global load and every wait on the copies is the
 //     explicit one below.
