@@ -163,10 +163,10 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     int nb_lo = n_wave >> 7, nb_hi = (n_wave + TN - 1) >> 7;
     nb_lo = nb_lo < sn ? nb_lo : sn - 1;
     nb_hi = nb_hi < sn ? nb_hi : sn - 1;
-    bool patch_hi[NJ];  // patch j lies in the second block
+    uint32_t hi_mask[NJ];  // all ones when patch j lies in the wave's second b_scale block
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
-        patch_hi[j] = ((n_wave + 32 * j) >> 7) > (n_wave >> 7);
+        hi_mask[j] = (uint32_t)-(int)(((n_wave + 32 * j) >> 7) > (n_wave >> 7));
 
     v16f acc[MI][NJ];
 #pragma unroll
@@ -268,8 +268,11 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
             }
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
-                // wave-uniform choice of the b_scale value (a scalar select), one product per patch
-                const float sc = sa[i] * (patch_hi[j] ? sb_hi : sb_lo);
+                // wave-uniform choice of the b_scale value on the scalar unit (bit select), then one
+                // product per patch
+                const float sbj = __uint_as_float((__float_as_uint(sb_hi) & hi_mask[j]) |
+                                                  (__float_as_uint(sb_lo) & ~hi_mask[j]));
+                const float sc = sa[i] * sbj;
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = fmaf(sc, blk[i][r], acc[i][j][r]);

@@ -170,10 +170,10 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
         int nb_lo = n_wave >> 7, nb_hi = (n_wave + TN - 1) >> 7;
         nb_lo = nb_lo < sn ? nb_lo : sn - 1;
         nb_hi = nb_hi < sn ? nb_hi : sn - 1;
-        bool patch_hi[NJ];
+        uint32_t hi_mask[NJ];  // all ones when patch jj lies in the wave's second b_scale block
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj)
-            patch_hi[jj] = ((n_wave + 32 * jj) >> 7) > (n_wave >> 7);
+            hi_mask[jj] = (uint32_t)-(int)(((n_wave + 32 * jj) >> 7) > (n_wave >> 7));
 
         v16f acc[MI][NJ];
 #pragma unroll
@@ -251,8 +251,11 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
                 }
 #pragma unroll
                 for (int i = 0; i < MI; ++i) {
-                    // wave-uniform choice of the b_scale value (a scalar select), one product per patch
-                    const float sc = sa[i] * (patch_hi[jj] ? sb_hi : sb_lo);
+                    // wave-uniform choice of the b_scale value on the scalar unit (bit select), then one
+                    // product per patch
+                    const float sbj = __uint_as_float((__float_as_uint(sb_hi) & hi_mask[jj]) |
+                                                      (__float_as_uint(sb_lo) & ~hi_mask[jj]));
+                    const float sc = sa[i] * sbj;
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
                         acc[i][jj][r] = fmaf(sc, blk[i][r], acc[i][jj][r]);
