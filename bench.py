@@ -231,7 +231,26 @@ def main():
             cold = cold_latency_us(dev, dc, shape)
             rep["cold_latency_us"] = round(cold, 2)
             rep["cold_gbs"] = round(byts / cold * 1e-3, 1)
+        if not args.no_cpu and not isinstance(name, tuple):
+            rep["cpu"] = cpu_row(shape, host)
         return rep, (shape, host, wall_ms, ev_ms)
+
+    def cpu_row(shape, host, max_rows=1024):
+        """the CPU oracle on the first rows of the same inputs, all host threads, best of up to 3"""
+        m_, n_, k_ = shape
+        rows = min(m_, max_rows)
+        a_s = np.ascontiguousarray(host[0][:, :rows])
+        sa_s = np.ascontiguousarray(host[2][:, :rows])
+        threads = oracle.max_threads()
+        best = None
+        for _ in range(3 if 2.0 * rows * n_ * k_ < 5e10 else 1):
+            t0 = time.perf_counter()
+            oracle.ref_gemm(a_s, host[1], sa_s, host[3], rows, n_, k_, nthreads=threads)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return {"rows": rows, "of_rows": m_, "threads": threads, "us": round(best * 1e6, 1),
+                "gflops": round(2.0 * rows * n_ * k_ / best * 1e-9, 1),
+                "full_shape_us_extrapolated": round(best * 1e6 * m_ / rows, 1)}
 
     def challenge_report(steps, warmup):
         rows = []
