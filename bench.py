@@ -323,6 +323,41 @@ def main():
         except Exception as exc:  # library or dtype not available: context only
             return {"what": "torch._scaled_mm unavailable", "error": repr(exc)[:200]}
 
+    def grouped_report(steps, warmup):
+        """cfg2's problem cut into eight groups of ragged M (an MoE layer's experts): one grouped
+        launch against eight launches of fp8_block_gemm_stream, same buffers"""
+        ms = [512, 1024, 768, 1536, 256, 2048, 1024, 1024]
+        gn, gk = 7168, 2048
+        bufs = []
+        for g, gm in enumerate(ms):
+            a_, b_, sa_, sb_ = oracle.make_inputs(gm, gn, gk, 5000 + g)
+            bufs.append([torch.from_numpy(x).cuda() for x in (a_, b_, sa_, sb_)] +
+                        [torch.zeros((gm, gn), dtype=torch.int16, device="cuda")])
+        cols = lambda i: [bf[i] for bf in bufs]
+        grouped = lambda: pkg.gemm_grouped(cols(0), cols(1), cols(2), cols(3), cols(4), ms, gn, gk, sptr)
+
+        def one_by_one():
+            for bf, gm in zip(bufs, ms):
+                pkg.gemm(bf[0], bf[1], bf[2], bf[3], bf[4], gm, gn, gk, sptr)
+
+        out = {"m": ms, "n": gn, "k": gk}
+        gflop = 2.0 * sum(ms) * gn * gk
+        for tag, fn in (("grouped", grouped), ("one_by_one", one_by_one)):
+            settle(fn, warmup)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / steps
+            out[tag + "_us"] = round(us, 2)
+            out[tag + "_tflops"] = round(gflop / us * 1e-6, 1)
+            if tag == "grouped":
+                out["kernel"] = pkg.last_kernel()
+        return out
+
     def launch_floor_us(reps=200):
         """back-to-back launches of a one-workgroup kernel of this library"""
         x = torch.zeros(256, dtype=torch.float32, device="cuda")
@@ -358,6 +393,7 @@ def main():
     floor_us = launch_floor_us()
     quantisers = None if args.no_shapes else quantiser_report(max(100, args.steps), args.warmup)
     vendor = None if args.no_shapes else vendor_plain_fp8_gemm_us(max(10, args.steps // 2), args.warmup)
+    grouped = None if args.no_shapes else grouped_report(max(30, args.steps), args.warmup)
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
               "max_sclk_mhz": max_sclk_mhz(),
@@ -419,6 +455,7 @@ def main():
         "challenge": challenge,
         "quantisers": quantisers,
         "vendor_plain_fp8_gemm": vendor,
+        "grouped": grouped,
         "device": device,
     }
     print(json.dumps(out))

@@ -60,6 +60,8 @@ def lib():
     L.fp8_block_gemm_select.argtypes = [i]
     L.fp8_block_gemm_force_config.restype = i
     L.fp8_block_gemm_force_config.argtypes = [i, i]
+    L.fp8_block_gemm_grouped.restype = i
+    L.fp8_block_gemm_grouped.argtypes = [i, vp, vp, vp, vp, vp, vp, i, i, vp]
     L.fp8_block_gemm_set_persistent.restype = i
     L.fp8_block_gemm_set_persistent.argtypes = [i]
     L.fp8_block_gemm_plan.restype = i
@@ -129,6 +131,18 @@ def select(kernel_id):
 
 def force_config(tile_variant=-1, ksplit=0):
     _check(lib().fp8_block_gemm_force_config(tile_variant, ksplit), "fp8_block_gemm_force_config")
+
+
+def gemm_grouped(a, b, a_scale, b_scale, c, m, n, k, stream=None):
+    """Grouped GEMM: lists of per-group tensors (or raw device pointers) and a list of per-group m;
+    all groups share n and k.  One persistent launch when every m is a multiple of 16."""
+    groups = len(m)
+    if not (len(a) == len(b) == len(a_scale) == len(b_scale) == len(c) == groups):
+        raise ValueError("one entry per group in every list")
+    ptrs = lambda xs: (C.c_void_p * groups)(*[_ptr(x) for x in xs])
+    ms = (C.c_int * groups)(*[int(v) for v in m])
+    _check(lib().fp8_block_gemm_grouped(groups, ptrs(a), ptrs(b), ptrs(a_scale), ptrs(b_scale), ptrs(c),
+                                        ms, n, k, stream), "fp8_block_gemm_grouped")
 
 
 def set_persistent(mode=-1):

@@ -296,6 +296,82 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit)
     return FP8GEMM_OK;
 }
 
+int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* b,
+                           const float* const* a_scale, const float* const* b_scale,
+                           void* const* c, const int* m, int n, int k, void* stream)
+{
+    if (groups < 0)
+        return FP8GEMM_E_SHAPE;
+    if (groups == 0)
+        return FP8GEMM_OK;
+    if (!a || !b || !a_scale || !b_scale || !c || !m)
+        return FP8GEMM_E_NULLPTR;
+    // every problem is validated before anything is launched
+    long long m_total = 0;
+    int live = 0;
+    for (int g = 0; g < groups; ++g) {
+        if (m[g] < 0)
+            return FP8GEMM_E_SHAPE;
+        if (m[g] == 0)
+            continue;
+        const int v = validate(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k);
+        if (v != FP8GEMM_OK)
+            return v;
+        m_total += m[g];
+        ++live;
+    }
+    if (live == 0)
+        return FP8GEMM_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    static_assert(GroupTable::MAX_GROUPS == FP8GEMM_MAX_GROUPS, "table size mirrors the ABI constant");
+    if (live <= GroupTable::MAX_GROUPS && g_selected.load() == FP8GEMM_KERNEL_AUTO && m_total <= 0x7FFFFFFFll) {
+        GroupTable tab;
+        tab.groups = 0;
+        for (int g = 0; g < groups; ++g) {
+            if (m[g] == 0)
+                continue;
+            const int t = tab.groups++;
+            tab.a[t] = static_cast<const uint8_t*>(a[g]);
+            tab.b[t] = static_cast<const uint8_t*>(b[g]);
+            tab.a_scale[t] = a_scale[g];
+            tab.b_scale[t] = b_scale[g];
+            tab.c[t] = static_cast<uint16_t*>(c[g]);
+            tab.m[t] = m[g];
+        }
+        // tile shape: what the cost model picks for the stacked problem, among the shapes that
+        // have a persistent form, without a K split
+        int best_v = -1;
+        double best = 1e300;
+        const int fv = g_force_variant.load();
+        GemmArgs stacked{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], (int)m_total, n, k};
+        for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
+            if ((fv >= 0 && v != fv) || !tile_grouped_supports(tab, n, k, v))
+                continue;
+            const double cst = tile_cost(stacked, v, 1);
+            if (cst < best) {
+                best = cst;
+                best_v = v;
+            }
+        }
+        if (best_v >= 0) {
+            const hipError_t e = launch_tile_grouped(tab, n, k, best_v, NUM_CU, s);
+            if (e == hipSuccess) {
+                snprintf(t_name_buf, sizeof(t_name_buf), "%s_k1_grouped%d", tile_variant_name(best_v), tab.groups);
+                t_last_kernel = t_name_buf;
+            }
+            return (int)e;
+        }
+    }
+    for (int g = 0; g < groups; ++g) {
+        if (m[g] == 0)
+            continue;
+        const int rc = run(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k, s, g_selected.load());
+        if (rc != FP8GEMM_OK)
+            return rc;
+    }
+    return FP8GEMM_OK;
+}
+
 int fp8_block_gemm_set_persistent(int mode)
 {
     if (mode < -1 || mode > 1)

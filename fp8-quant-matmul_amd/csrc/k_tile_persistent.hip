@@ -22,11 +22,21 @@ namespace fp8gemm {
 
 namespace {
 
-template <int BM, int BN, int WM, int WN, int NS, int PR>
-__global__ void __launch_bounds__(NTHREADS)
-tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
-                            const float* __restrict__ a_scale, const float* __restrict__ b_scale,
-                            uint16_t* __restrict__ c, int M, int N, int K, int tiles_m, int tiles_n)
+// One problem of a grouped launch as the kernel sees it.
+struct Problem {
+    const uint8_t* a;
+    const uint8_t* b;
+    const float* a_scale;
+    const float* b_scale;
+    uint16_t* c;
+    int M;
+};
+
+// GROUPED = false: one problem (`one`), tiles_m x tiles_n tiles.  GROUPED = true: the problems of
+// `tab` (same N and K, own M), whose tiles are numbered one group after the other.
+template <int BM, int BN, int WM, int WN, int NS, int PR, bool GROUPED>
+__device__ __forceinline__ void persistent_body(const Problem& one, const GroupTable* tab, int N, int K,
+                                                int tiles_m, int tiles_n)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
     static_assert(WM * WN == 8, "eight waves per workgroup");
@@ -53,7 +63,7 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
     // a contiguous run of the tile order (groups of GROUP_M tile rows, as in k_tile.hip) and
     // its workgroups take the run's tiles in turn, so that the tiles an XCD works on at any
     // moment are neighbours and share A and B panels in its L2.
-    const int T = tiles_m * tiles_n;
+    const int T = GROUPED ? tab->tile_start[tab->groups] : tiles_m * tiles_n;
     const int pid = blockIdx.x, per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
     const int xcd = pid & 7, q8 = T >> 3, r8 = T & 7;
     const int run0 = xcd * q8 + (xcd < r8 ? xcd : r8);
@@ -63,11 +73,23 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
     if (n_my == 0)
         return;
     const int per_group = GROUP_M * tiles_n;
-    auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {
-        const int logical = run0 + li + j * per_xcd;
+    // tile number j of this workgroup: its problem and its origin in that problem's C
+    auto tile_origin = [&](int j, Problem& pr, int& m0, int& n0) __attribute__((always_inline)) {
+        int logical = run0 + li + j * per_xcd;
+        int tm = tiles_m;
+        if (GROUPED) {
+            int g = 0;
+            while (g + 1 < tab->groups && logical >= tab->tile_start[g + 1])
+                ++g;
+            logical -= tab->tile_start[g];
+            pr = Problem{tab->a[g], tab->b[g], tab->a_scale[g], tab->b_scale[g], tab->c[g], tab->m[g]};
+            tm = (pr.M + BM - 1) / BM;
+        } else {
+            pr = one;
+        }
         const int group = logical / per_group;
         const int first_m = group * GROUP_M;
-        const int gsz = (tiles_m - first_m < GROUP_M) ? (tiles_m - first_m) : GROUP_M;
+        const int gsz = (tm - first_m < GROUP_M) ? (tm - first_m) : GROUP_M;
         const int in_group = logical - group * per_group;
         m0 = (first_m + in_group % gsz) * BM;
         n0 = (in_group / gsz) * BN;
@@ -75,10 +97,15 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
 
     const int nkb = K / KBLOCK;
     const int sn = (N + KBLOCK - 1) / KBLOCK;
-    const uint32_t a_bytes = (uint32_t)M * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
-    const uint32_t as_bytes = (uint32_t)nkb * (uint32_t)M * 4u;
-    const v4i rsrc_a = make_rsrc_words(a, a_bytes), rsrc_b = make_rsrc_words(b, b_bytes);
-    const v4i rsrc_s = make_rsrc_words(a_scale, as_bytes);
+    // buffer resources of the copy stream's current tile (fixed for a single problem)
+    v4i rsrc_a, rsrc_b, rsrc_s;
+    int f_M = one.M;  // rows of the problem the copy stream is in
+    auto set_resources = [&](const Problem& pr) __attribute__((always_inline)) {
+        rsrc_a = make_rsrc_words(pr.a, (uint32_t)pr.M * (uint32_t)K);
+        rsrc_b = make_rsrc_words(pr.b, (uint32_t)N * (uint32_t)K);
+        rsrc_s = make_rsrc_words(pr.a_scale, (uint32_t)nkb * (uint32_t)pr.M * 4u);
+        f_M = pr.M;
+    };
 
     // ---- the copy stream: K block f_kb of this workgroup's tile number f_tile is the next one
     // to be copied.  Per-lane offsets (copy plan of k_tile.hip) belong to that tile.
@@ -86,8 +113,12 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
     int f_tile = 0, f_kb = 0;
     int fill_left = n_my * nkb;  // blocks not yet copied
     auto fill_setup = [&](int j) __attribute__((always_inline)) {
+        Problem pr;
         int m0, n0;
-        tile_origin(j, m0, n0);
+        tile_origin(j, pr, m0, n0);
+        if (GROUPED || j == 0)
+            set_resources(pr);
+        const int M = pr.M;
 #pragma unroll
         for (int q = 0; q < S::NVA; ++q) {
             const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
@@ -109,13 +140,13 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
         const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
         if (q < NA) {
             lds_dma16(rsrc_a, voff_a[S::template voff_index<RSA>(q)], stage + (uint32_t)((NA * wave + q) * 1024),
-                      (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)M);
+                      (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)f_M);
         } else if (q < NA + NB) {
             lds_dma16(rsrc_b, voff_b[S::template voff_index<RSB>(q - NA)],
                       stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
                       (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSB>(q - NA)) * (uint32_t)N);
         } else if (wave == 0) {
-            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)f_kb * (uint32_t)M * 4u);
+            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)f_kb * (uint32_t)f_M * 4u);
         }
     };
     auto fill_advance = [&]() __attribute__((always_inline)) {
@@ -164,8 +195,12 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
     int slot_fill = NS - 1;  // ring slot the stream's next block goes into
 
     for (int j = 0; j < n_my; ++j) {
+        Problem pr;
         int m0, n0;
-        tile_origin(j, m0, n0);
+        tile_origin(j, pr, m0, n0);
+        const float* __restrict__ b_scale = pr.b_scale;
+        uint16_t* __restrict__ c = pr.c;
+        const int M = pr.M;
         const int n_wave = n0 + wn * TN;
         int nb_lo = n_wave >> 7, nb_hi = (n_wave + TN - 1) >> 7;
         nb_lo = nb_lo < sn ? nb_lo : sn - 1;
@@ -331,6 +366,24 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
 }
 
 template <int BM, int BN, int WM, int WN, int NS, int PR>
+__global__ void __launch_bounds__(NTHREADS)
+tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                            const float* __restrict__ a_scale, const float* __restrict__ b_scale,
+                            uint16_t* __restrict__ c, int M, int N, int K, int tiles_m, int tiles_n)
+{
+    const Problem one{a, b, a_scale, b_scale, c, M};
+    persistent_body<BM, BN, WM, WN, NS, PR, false>(one, nullptr, N, K, tiles_m, tiles_n);
+}
+
+template <int BM, int BN, int WM, int WN, int NS, int PR>
+__global__ void __launch_bounds__(NTHREADS)
+tile_gemm_grouped_kernel(const GroupTable tab, int N, int K, int tiles_n)
+{
+    const Problem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    persistent_body<BM, BN, WM, WN, NS, PR, true>(none, &tab, N, K, 0, tiles_n);
+}
+
+template <int BM, int BN, int WM, int WN, int NS, int PR>
 hipError_t launch_persistent_variant(const GemmArgs& g, int workgroups, hipStream_t s)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
@@ -346,19 +399,41 @@ hipError_t launch_persistent_variant(const GemmArgs& g, int workgroups, hipStrea
     return hipGetLastError();
 }
 
+template <int BM, int BN, int WM, int WN, int NS, int PR>
+hipError_t launch_grouped_variant(GroupTable& tab, int n, int k, int workgroups, hipStream_t s)
+{
+    using S = TileShape<BM, BN, WM, WN, NS>;
+    constexpr int LDS_TOTAL = S::LDS_BYTES;
+    const int tiles_n = (n + BN - 1) / BN;
+    tab.tile_start[0] = 0;
+    for (int g = 0; g < tab.groups; ++g)
+        tab.tile_start[g + 1] = tab.tile_start[g] + ((tab.m[g] + BM - 1) / BM) * tiles_n;
+    auto kern = tile_gemm_grouped_kernel<BM, BN, WM, WN, NS, PR>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
+    if (e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kern, dim3(workgroups), dim3(NTHREADS), LDS_TOTAL, s, tab, n, k, tiles_n);
+    return hipGetLastError();
+}
+
+int persistent_stages(int variant)
+{
+    switch (variant) {
+    case TILE_256x192: return 2;
+    case TILE_256x128: return 3;
+    case TILE_128x192: return 3;
+    case TILE_128x128: return 4;
+    default: return 0;
+    }
+}
+
 }  // namespace
 
 bool tile_persistent_supports(const GemmArgs& g, int variant)
 {
-    int stages;
-    switch (variant) {
-    case TILE_256x192: stages = 2; break;
-    case TILE_256x128: stages = 3; break;
-    case TILE_128x192: stages = 3; break;
-    case TILE_128x128: stages = 4; break;
-    default: return false;
-    }
-    return tile_supports(g) && g.k / KBLOCK >= stages - 1;
+    const int stages = persistent_stages(variant);
+    return stages > 0 && tile_supports(g) && g.k / KBLOCK >= stages - 1;
 }
 
 hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups, hipStream_t s)
@@ -370,6 +445,33 @@ hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups
     case TILE_256x128: return launch_persistent_variant<256, 128, 4, 2, 3, 128>(g, workgroups, s);
     case TILE_128x192: return launch_persistent_variant<128, 192, 4, 2, 3, 128>(g, workgroups, s);
     case TILE_128x128: return launch_persistent_variant<128, 128, 2, 4, 4, 128>(g, workgroups, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// every group non-empty, aligned like a single problem, K long enough for the ring
+bool tile_grouped_supports(const GroupTable& tab, int n, int k, int variant)
+{
+    const int stages = persistent_stages(variant);
+    if (stages == 0 || k / KBLOCK < stages - 1 || tab.groups < 1 || tab.groups > GroupTable::MAX_GROUPS)
+        return false;
+    for (int g = 0; g < tab.groups; ++g) {
+        const GemmArgs ga{tab.a[g], tab.b[g], tab.a_scale[g], tab.b_scale[g], tab.c[g], tab.m[g], n, k};
+        if (tab.m[g] <= 0 || !tile_supports(ga))
+            return false;
+    }
+    return true;
+}
+
+hipError_t launch_tile_grouped(GroupTable& tab, int n, int k, int variant, int workgroups, hipStream_t s)
+{
+    if (workgroups <= 0 || workgroups % 8 != 0 || !tile_grouped_supports(tab, n, k, variant))
+        return hipErrorInvalidValue;
+    switch (variant) {
+    case TILE_256x192: return launch_grouped_variant<256, 192, 4, 2, 2, 128>(tab, n, k, workgroups, s);
+    case TILE_256x128: return launch_grouped_variant<256, 128, 4, 2, 3, 128>(tab, n, k, workgroups, s);
+    case TILE_128x192: return launch_grouped_variant<128, 192, 4, 2, 3, 128>(tab, n, k, workgroups, s);
+    case TILE_128x128: return launch_grouped_variant<128, 128, 2, 4, 4, 128>(tab, n, k, workgroups, s);
     default: return hipErrorInvalidValue;
     }
 }

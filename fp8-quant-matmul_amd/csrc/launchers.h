@@ -32,6 +32,21 @@ hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partia
 // all tiles, the copies of a tile's first K blocks overlap the previous tile's epilogue.
 bool tile_persistent_supports(const GemmArgs& g, int variant);
 hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups, hipStream_t s);
+// Grouped form: several problems with the same n and k and their own m in one persistent launch
+// (the table travels by value in the kernel arguments; tile_start is filled by the launcher).
+struct GroupTable {
+    static constexpr int MAX_GROUPS = 64;
+    const uint8_t* a[MAX_GROUPS];
+    const uint8_t* b[MAX_GROUPS];
+    const float* a_scale[MAX_GROUPS];
+    const float* b_scale[MAX_GROUPS];
+    uint16_t* c[MAX_GROUPS];
+    int m[MAX_GROUPS];
+    int tile_start[MAX_GROUPS + 1];
+    int groups;
+};
+bool tile_grouped_supports(const GroupTable& tab, int n, int k, int variant);
+hipError_t launch_tile_grouped(GroupTable& tab, int n, int k, int variant, int workgroups, hipStream_t s);
 hipError_t launch_splitk_reduce(const GemmArgs& g, int ksplit, const float* partial, hipStream_t s);
 
 // tiny-M streaming kernel (decode shapes)

@@ -89,6 +89,20 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit);
  * allows.  The reference names such a kernel as future work (/root/reference/README.md:29). */
 int fp8_block_gemm_set_persistent(int mode);
 
+/* Grouped GEMM: `groups` independent problems with the same n and k and their own m[g]
+ * (ragged M, e.g. the experts of one MoE layer), C[g] = A[g] . B[g]^T with the layouts above.
+ * a, b, a_scale, b_scale, c and m are HOST arrays of `groups` entries; the pointers they hold
+ * are device pointers.  Groups with m[g] == 0 are skipped.  Up to FP8GEMM_MAX_GROUPS problems
+ * whose m[g] are multiples of 16 run as ONE launch of the persistent tile kernel (their tiles
+ * form one list that 256 workgroups walk through); anything else falls back to one call of
+ * fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to what
+ * fp8_block_gemm_stream gives for that problem with the same tile shape.  No counterpart in the
+ * reference, which launches one problem at a time (/root/reference/check.cu:106-114). */
+#define FP8GEMM_MAX_GROUPS 64
+int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* b,
+                           const float* const* a_scale, const float* const* b_scale,
+                           void* const* c, const int* m, int n, int k, void* stream);
+
 /* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
  * 16-byte aligned operands into name[0..cap), e.g. "tile256x256_k1", "skinny_k1", "scalar".
  * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart

@@ -10,7 +10,7 @@ import pytest
 def test_library_exports_every_declared_symbol(pkg):
     L = pkg.lib()
     names = pkg.abi_symbols()
-    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and len(names) >= 16
+    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and len(names) == 18
     for name in names:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
     assert L.fp8_block_gemm_abi_version() == 2
@@ -39,6 +39,23 @@ def test_argument_validation_happens_before_any_device_call(pkg):
         assert fn(p, 0, p, p, 70000, 65536, None) == -5
         assert fn(p, 7, p, p, 16, 128, None) == -6
         assert fn(p + 2, 0, p, p, 16, 128, None) == -7
+
+
+def test_grouped_entry_point_validates_every_group_first(pkg):
+    L = pkg.lib()
+    p = 4096
+    arr = lambda *v: (C.c_void_p * len(v))(*v)
+    ints = lambda *v: (C.c_int * len(v))(*v)
+    ok = arr(p, p)
+    assert L.fp8_block_gemm_grouped(-1, ok, ok, ok, ok, ok, ints(16, 16), 16, 128, None) == -2
+    assert L.fp8_block_gemm_grouped(0, None, None, None, None, None, None, 16, 128, None) == 0
+    assert L.fp8_block_gemm_grouped(2, ok, ok, ok, ok, ok, None, 16, 128, None) == -1
+    assert L.fp8_block_gemm_grouped(2, ok, ok, ok, ok, ok, ints(0, 0), 16, 128, None) == 0      # nothing to do
+    assert L.fp8_block_gemm_grouped(2, ok, arr(p, None), ok, ok, ok, ints(16, 16), 16, 128, None) == -1
+    assert L.fp8_block_gemm_grouped(2, ok, arr(p, None), ok, ok, ok, ints(16, 0), 16, 100, None) == -2
+    assert L.fp8_block_gemm_grouped(2, ok, ok, ok, ok, ok, ints(16, -4), 16, 128, None) == -2
+    with pytest.raises(ValueError):
+        pkg.gemm_grouped([p], [p, p], [p], [p], [p], [16], 16, 128)
 
 
 def test_error_strings_and_exception(pkg):

@@ -314,3 +314,55 @@ def test_custom_kernel_operator_form(pkg):
         pkg.custom_kernel((ta.contiguous(), tb, tsa, tsb, c))            # row-major a is refused
     with pytest.raises(ValueError):
         pkg.custom_kernel((ta, tb, tsa, tsb, c.t()))
+
+
+# ------------------------------------------------------------------ grouped GEMM
+def _grouped_case(pkg, ms, n, k, variant, seed):
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    host, dev, outs = [], [], []
+    for g, m in enumerate(ms):
+        mm = max(m, 16)                       # an empty group still gets valid (unused) buffers
+        a, b, sa, sb = oracle.make_inputs(mm, n, k, seed + 17 * g)
+        host.append((a, b, sa, sb))
+        dev.append(_dev(a, b, sa, sb))
+        outs.append(torch.full((mm, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16))
+    _say(f"[gpu case] grouped ms={ms} n={n} k={k} variant={variant}")
+    pkg.force_config(variant, 0)
+    try:
+        pkg.gemm_grouped([d[0] for d in dev], [d[1] for d in dev], [d[2] for d in dev], [d[3] for d in dev],
+                         outs, ms, n, k, st)
+        torch.cuda.synchronize()
+        name = pkg.last_kernel()
+    finally:
+        pkg.force_config(-1, 0)
+    return host, dev, outs, name
+
+
+@pytest.mark.parametrize("variant,ms,n,k", [(2, [256, 16, 1040, 0, 512], 576, 768),
+                                            (0, [4096, 272, 2048, 1024, 16], 1536, 512),
+                                            (1, [512] * 9 + [48, 2064], 1024, 384),
+                                            (3, [144] * 40, 384, 640),
+                                            (2, [128], 128, 384)])
+def test_grouped_gemm_equals_the_problems_one_by_one(pkg, variant, ms, n, k):
+    host, dev, outs, name = _grouped_case(pkg, ms, n, k, variant, 7000 + n + k)
+    assert "_grouped" in name, name
+    for g, m in enumerate(ms):
+        if m == 0:
+            assert (outs[g].cpu().numpy().view(np.uint16) == 0x7FC1).all()      # untouched
+            continue
+        a, b, sa, sb = host[g]
+        got = outs[g].cpu().numpy().view(np.uint16)
+        ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+        _assert_close(got, ref, f"{name} group {g}")
+        single, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant, persistent=0)
+        assert np.array_equal(got, single), f"group {g}: grouped launch and single launch differ"
+
+
+def test_grouped_gemm_falls_back_for_unaligned_groups(pkg):
+    ms, n, k = [40, 256, 24], 256, 256       # 40 and 24 rows: not multiples of 16
+    host, dev, outs, name = _grouped_case(pkg, ms, n, k, -1, 8100)
+    assert "_grouped" not in name, name
+    for g, m in enumerate(ms):
+        a, b, sa, sb = host[g]
+        _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
