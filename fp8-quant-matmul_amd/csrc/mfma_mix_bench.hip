@@ -119,7 +119,10 @@ int main(int argc, char** argv)
     run<0, 0>(d, out, iters);
     run<8, 0>(d, out, iters);
     run<0, 3>(d, out, iters);
+    run<8, 2>(d, out, iters);
     run<8, 3>(d, out, iters);
+    run<9, 2>(d, out, iters);
+    run<9, 3>(d, out, iters);
     run<10, 3>(d, out, iters);
     run<10, 4>(d, out, iters);
     run<12, 4>(d, out, iters);
