@@ -121,3 +121,12 @@ def test_dispatcher_plans(pkg):
 def test_header_cites_reference_for_every_entry_point(pkg):
     hdr = open(os.path.join(os.path.dirname(pkg.lib_path()), "..", "include", "fp8_block_gemm.h")).read()
     assert hdr.count("/root/reference/") >= 8
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
