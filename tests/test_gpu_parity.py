@@ -366,3 +366,23 @@ def test_grouped_gemm_falls_back_for_unaligned_groups(pkg):
     for g, m in enumerate(ms):
         a, b, sa, sb = host[g]
         _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
+
+
+def test_seeded_sweep_of_shapes_and_plans(pkg):
+    """forty pseudo-random (shape, tile, K split, persistence) combinations against the oracle"""
+    rs = np.random.RandomState(20241125)
+    for case in range(40):
+        m = int(rs.randint(1, 48)) * 16
+        n = int(rs.randint(1, 48)) * 16
+        k = int(rs.randint(1, 13)) * 128
+        variant = int(rs.randint(-1, 5))
+        nkb = k // 128
+        ksplit = int(rs.choice([0, 1, 1, 2, 3, 5])) if nkb >= 5 else int(rs.choice([0, 1]))
+        if ksplit > 1 and (ksplit - 1) * -(-nkb // ksplit) >= nkb:
+            ksplit = 0                        # a split without a K block of its own: not a valid pin
+        persistent = int(rs.randint(-1, 2))
+        a, b, sa, sb = oracle.make_inputs(m, n, k, 9000 + case, 0.5, 20.0)
+        ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+        got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_AUTO, variant=variant, ksplit=ksplit,
+                         persistent=persistent)
+        _assert_close(got, ref, f"case {case}: m={m} n={n} k={k} -> {name}")
