@@ -104,7 +104,7 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
                            void* const* c, const int* m, int n, int k, void* stream);
 
 /* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
- * 16-byte aligned operands into name[0..cap), e.g. "tile256x256_k1", "skinny_k1", "scalar".
+ * 16-byte aligned operands into name[0..cap), e.g. "tile256x192_k1_persistent", "tile128x128_k3", "skinny_k1", "scalar".
  * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart
  * in the reference (its choice is made by editing the source, README.md:55). */
 int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap);
