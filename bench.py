@@ -323,6 +323,28 @@ def main():
         except Exception as exc:  # library or dtype not available: context only
             return {"what": "torch._scaled_mm unavailable", "error": repr(exc)[:200]}
 
+    def host_boundary_report():
+        """fp8_gemm_host on the headline shape: host fp32 values in, bf16 out, device memory
+        allocated, filled over PCIe, converted, multiplied, read back and freed inside the call
+        (pageable host memory, as the reference's harness uses).  Never `value`."""
+        ha, hb, sa, sb = host
+        af, bf = oracle.e4m3fn_decode(ha), oracle.e4m3fn_decode(hb)
+        ch = np.zeros((m, n), np.uint16)
+        L = pkg.lib()
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            rc = L.fp8_gemm_host(ch.ctypes.data, af.ctypes.data, bf.ctypes.data, sa.ctypes.data,
+                                 sb.ctypes.data, m, n, k, 0)
+            dt = time.perf_counter() - t0
+            if rc != 0:
+                return {"error": rc}
+            best = dt if best is None else min(best, dt)
+        moved = af.nbytes + bf.nbytes + sa.nbytes + sb.nbytes + ch.nbytes
+        return {"what": "fp8_gemm_host, best of 3: alloc + PCIe in (fp32 values) + convert + GEMM + PCIe out + free",
+                "ms": round(best * 1e3, 2), "tflops": round(flops / best * 1e-12, 2),
+                "host_bytes_moved": moved, "host_gbs": round(moved / best * 1e-9, 1)}
+
     def grouped_report(steps, warmup):
         """cfg2's problem cut into eight groups of ragged M (an MoE layer's experts): one grouped
         launch against eight launches of fp8_block_gemm_stream, same buffers"""
@@ -394,6 +416,7 @@ def main():
     quantisers = None if args.no_shapes else quantiser_report(max(100, args.steps), args.warmup)
     vendor = None if args.no_shapes else vendor_plain_fp8_gemm_us(max(10, args.steps // 2), args.warmup)
     grouped = None if args.no_shapes else grouped_report(max(30, args.steps), args.warmup)
+    host_boundary = None if args.no_shapes else host_boundary_report()
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
               "max_sclk_mhz": max_sclk_mhz(),
@@ -453,6 +476,7 @@ def main():
         "quantisers": quantisers,
         "vendor_plain_fp8_gemm": vendor,
         "grouped": grouped,
+        "host_boundary": host_boundary,
         "device": device,
     }
     print(json.dumps(out))
