@@ -408,12 +408,12 @@ size_t fp8_block_gemm_workspace_bytes(int m, int n, int k)
 {
     if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
         return 0;
-    // upper bound over every plan the dispatcher can pick: at most 16 K splits (64 when
-    // forced), each an m x n fp32 partial
-    int ks = g_force_ksplit.load() > 16 ? g_force_ksplit.load() : 16;
-    if (ks > k / 128)
-        ks = k / 128;
-    return (size_t)ks * m * n * sizeof(float);
+    // what the plan for 16-byte aligned operands needs under the current selection and forced
+    // configuration; operands with less alignment run kernels that need the same or nothing
+    GemmArgs g{reinterpret_cast<const uint8_t*>(uintptr_t(4096)), reinterpret_cast<const uint8_t*>(uintptr_t(4096)),
+               nullptr, nullptr, reinterpret_cast<uint16_t*>(uintptr_t(4096)), m, n, k};
+    const Plan p = make_plan(g, g_selected.load());
+    return p.family < 0 ? 0 : plan_workspace_bytes(g, p);
 }
 
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)

@@ -115,10 +115,15 @@ const char* fp8_block_gemm_last_kernel(void);
 
 /* Split-K kernels keep fp32 partial tiles in device memory.  By default the library owns a
  * lazily grown buffer (allocated on first need, kept until fp8_block_gemm_release).
- * A caller that must not allocate can supply its own: `bytes` must be at least
- * fp8_block_gemm_workspace_bytes(m, n, k) for every later call, 256-byte aligned.
- * Passing NULL returns to the library-owned buffer.  The reference has no workspace
- * (its kernels do not split K: mn_small.hip:28). */
+ * A caller that must not allocate can supply its own, 256-byte aligned, of at least
+ * fp8_block_gemm_workspace_bytes(m, n, k) bytes for every shape it will pass: that is what
+ * the plan for the shape needs under the kernel selection and forced configuration in force
+ * when it is asked (0 when the plan does not split K; ask again after changing either).
+ * Passing NULL returns to the library-owned buffer.  There is ONE workspace per process,
+ * on the device that was current when it was allocated or supplied: calls that split K
+ * (fp8_block_gemm_plan names them "..._kN" with N > 1) must not overlap on different streams,
+ * and must run on that device; calls that do not split K never touch it.  The reference has
+ * no workspace (its kernels do not split K: mn_small.hip:28). */
 size_t fp8_block_gemm_workspace_bytes(int m, int n, int k);
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes);
 int fp8_block_gemm_release(void);

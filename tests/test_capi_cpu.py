@@ -91,8 +91,15 @@ def test_select_and_force_config_validate(pkg):
 def test_workspace_contract(pkg):
     L = pkg.lib()
     assert pkg.workspace_bytes(0, 8, 128) == 0
-    assert pkg.workspace_bytes(64, 64, 128) == 64 * 64 * 4          # one K block: no split beyond 1
-    assert pkg.workspace_bytes(1024, 512, 2048) == 16 * 1024 * 512 * 4
+    assert pkg.workspace_bytes(64, 64, 128) == 0                     # one K block: nothing to split
+    assert pkg.workspace_bytes(8192, 4608, 7168) == 0                # plan does not split K
+    assert pkg.plan(1024, 512, 7168) == "tile128x128_k6"
+    assert pkg.workspace_bytes(1024, 512, 7168) == 6 * 1024 * 512 * 4
+    assert L.fp8_block_gemm_force_config(2, 8) == 0                  # follows a forced configuration
+    try:
+        assert pkg.workspace_bytes(256, 256, 1024) == 8 * 256 * 256 * 4
+    finally:
+        assert L.fp8_block_gemm_force_config(-1, 0) == 0
     assert L.fp8_block_gemm_set_workspace(4096 + 8, 1 << 20) == -4   # misaligned
     assert L.fp8_block_gemm_set_workspace(None, 0) == 0
     assert L.fp8_block_gemm_release() == 0                           # nothing allocated yet

@@ -264,7 +264,14 @@ def test_caller_workspace(pkg):
     m, n, k = 256, 256, 1024
     a, b, sa, sb = oracle.make_inputs(m, n, k, 62)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
-    need = pkg.workspace_bytes(m, n, k)
+    pkg.select(3)
+    pkg.force_config(2, 8)
+    try:
+        need = pkg.workspace_bytes(m, n, k)
+    finally:
+        pkg.force_config(-1, 0)
+        pkg.select(0)
+    assert need == 8 * m * n * 4
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     pkg.set_workspace(ws, need)
     try:
