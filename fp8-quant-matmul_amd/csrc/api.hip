@@ -34,7 +34,46 @@ struct Plan {
     int variant;  // TileVariant for the tile families
     int ksplit;
     bool persistent = false;  // tile families, ksplit == 1: workgroups walk through the tiles
+    bool padded = false;      // the plan is for the problem with m and n rounded up to 16 (run_padded)
 };
+
+// Shapes or addresses the MFMA kernels cannot take (m or n not a multiple of 16, a base not
+// 16-byte aligned) run on padded copies in the workspace: which operands are copied, and where.
+struct PadLayout {
+    bool a, as, b, c;
+    int m16, n16;
+    size_t off_a, off_as, off_b, off_c, off_partial, total;
+};
+
+inline size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
+inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; }
+
+// conservative = true: every operand copied (an upper bound that does not depend on addresses)
+PadLayout pad_layout(const GemmArgs& g, size_t partial_bytes, bool conservative)
+{
+    PadLayout L{};
+    L.m16 = (g.m + 15) & ~15;
+    L.n16 = (g.n + 15) & ~15;
+    const bool rm = L.m16 != g.m, rn = L.n16 != g.n;
+    L.a = conservative || rm || misaligned16(g.a);
+    L.as = conservative || rm || misaligned16(g.a_scale);
+    L.b = conservative || rn || misaligned16(g.b);
+    L.c = conservative || rm || rn || misaligned16(g.c);
+    const size_t nkb = (size_t)g.k / 128;
+    size_t off = 0;
+    L.off_a = off;
+    off += L.a ? round256((size_t)g.k * L.m16) : 0;
+    L.off_as = off;
+    off += L.as ? round256(nkb * L.m16 * sizeof(float)) : 0;
+    L.off_b = off;
+    off += L.b ? round256((size_t)g.k * L.n16) : 0;
+    L.off_c = off;
+    off += L.c ? round256((size_t)L.m16 * L.n16 * 2) : 0;
+    L.off_partial = off;
+    off += partial_bytes;
+    L.total = off;
+    return L;
+}
 
 int validate(const void* a, const void* b, const float* as, const float* bs, const void* c, int m,
              int n, int k)
@@ -110,9 +149,22 @@ Plan make_plan(const GemmArgs& g, int selected)
         }
     }
     if (!tile_supports(g)) {
-        if (selected != FP8GEMM_KERNEL_AUTO)
+        if (selected != FP8GEMM_KERNEL_AUTO) {
             p.family = -1;
-        return p;  // scalar fallback for shapes without 16-byte row alignment
+            return p;
+        }
+        // rows without 16-byte alignment: the padded problem (its four extra launches cost
+        // about 12 us; the scalar kernel, one dependent load after the other, takes 30 us for
+        // K = 128 already), unless padding pushes an operand past the size limit
+        const long long m16 = (g.m + 15) & ~15, n16 = (g.n + 15) & ~15, lim = 0x7FFFFFFFll;
+        if (m16 * g.k > lim || n16 * g.k > lim || m16 * n16 > lim)
+            return p;
+        const uint8_t* const al8 = reinterpret_cast<const uint8_t*>(uintptr_t(4096));
+        GemmArgs gp{al8, al8, reinterpret_cast<const float*>(uintptr_t(4096)), g.b_scale,
+                    reinterpret_cast<uint16_t*>(uintptr_t(4096)), (int)m16, (int)n16, g.k};
+        p = make_plan(gp, selected);
+        p.padded = p.family != FP8GEMM_KERNEL_SCALAR && p.family >= 0;
+        return p;
     }
     const int fv = g_force_variant.load(), fk = g_force_ksplit.load();
     const int nkb = g.k / 128;
@@ -201,6 +253,73 @@ size_t plan_workspace_bytes(const GemmArgs& g, const Plan& p)
     return (size_t)p.ksplit * g.m * g.n * sizeof(float);
 }
 
+void plan_name(const Plan& p, char* out, size_t cap)
+{
+    const char* pre = p.padded ? "padded_" : "";
+    if (p.family == FP8GEMM_KERNEL_SCALAR)
+        snprintf(out, cap, "scalar");
+    else if (p.family == FP8GEMM_KERNEL_SKINNY)
+        snprintf(out, cap, "%sskinny_k%d", pre, p.ksplit);
+    else
+        snprintf(out, cap, "%s%s_k%d%s", pre, tile_variant_name(p.variant), p.ksplit,
+                 p.persistent ? "_persistent" : "");
+}
+
+// the kernels of a plan on operands they can take; `partial` holds plan_workspace_bytes
+hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, hipStream_t stream)
+{
+    switch (p.family) {
+    case FP8GEMM_KERNEL_SCALAR:
+        return launch_scalar(g, stream);
+    case FP8GEMM_KERNEL_SKINNY:
+        return launch_skinny(g, partial, stream);
+    default: {
+        if (p.persistent)
+            return launch_tile_persistent(g, p.variant, NUM_CU, stream);
+        hipError_t e = launch_tile(g, p.variant, p.ksplit, partial, stream);
+        if (e == hipSuccess && p.ksplit > 1)
+            e = launch_splitk_reduce(g, p.ksplit, partial, stream);
+        return e;
+    }
+    }
+}
+
+// pad what needs padding into the workspace, run the plan there, copy C's corner out
+int run_padded(const GemmArgs& g, const Plan& p, hipStream_t stream)
+{
+    GemmArgs gp = g;
+    gp.m = (g.m + 15) & ~15;
+    gp.n = (g.n + 15) & ~15;
+    const PadLayout L = pad_layout(g, plan_workspace_bytes(gp, p), false);
+    int err;
+    float* ws = get_workspace(L.total, &err);
+    if (!ws)
+        return err;
+    uint8_t* base = reinterpret_cast<uint8_t*>(ws);
+    const int nkb = g.k / 128;
+    hipError_t e = hipSuccess;
+    if (L.a) {
+        e = launch_pad_bytes(g.a, base + L.off_a, g.k, g.m, gp.m, stream);
+        gp.a = base + L.off_a;
+    }
+    if (e == hipSuccess && L.as) {
+        float* as = reinterpret_cast<float*>(base + L.off_as);
+        e = launch_pad_floats(g.a_scale, as, nkb, g.m, gp.m, stream);
+        gp.a_scale = as;
+    }
+    if (e == hipSuccess && L.b) {
+        e = launch_pad_bytes(g.b, base + L.off_b, g.k, g.n, gp.n, stream);
+        gp.b = base + L.off_b;
+    }
+    if (L.c)
+        gp.c = reinterpret_cast<uint16_t*>(base + L.off_c);
+    if (e == hipSuccess)
+        e = launch_plan(gp, p, reinterpret_cast<float*>(base + L.off_partial), stream);
+    if (e == hipSuccess && L.c)
+        e = launch_crop_bf16(gp.c, g.c, g.m, g.n, gp.n, stream);
+    return (int)e;
+}
+
 int run(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k,
         hipStream_t stream, int selected)
 {
@@ -209,50 +328,26 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
         return v;
     GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), as, bs,
                static_cast<uint16_t*>(c), m, n, k};
-    Plan p = make_plan(g, selected);
+    const Plan p = make_plan(g, selected);
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
-    hipError_t e = hipSuccess;
-    switch (p.family) {
-    case FP8GEMM_KERNEL_SCALAR:
-        e = launch_scalar(g, stream);
-        t_last_kernel = "scalar";
-        break;
-    case FP8GEMM_KERNEL_SKINNY: {
+    int rc;
+    if (p.padded) {
+        rc = run_padded(g, p, stream);
+    } else {
         float* ws = nullptr;
-        if (p.ksplit > 1) {
+        const size_t need = plan_workspace_bytes(g, p);
+        if (need) {
             int err;
-            ws = get_workspace(plan_workspace_bytes(g, p), &err);
+            ws = get_workspace(need, &err);
             if (!ws)
                 return err;
         }
-        e = launch_skinny(g, ws, stream);
-        snprintf(t_name_buf, sizeof(t_name_buf), "skinny_k%d", p.ksplit);
-        t_last_kernel = t_name_buf;
-        break;
+        rc = (int)launch_plan(g, p, ws, stream);
     }
-    default: {
-        float* ws = nullptr;
-        if (p.ksplit > 1) {
-            int err;
-            ws = get_workspace(plan_workspace_bytes(g, p), &err);
-            if (!ws)
-                return err;
-        }
-        if (p.persistent) {
-            e = launch_tile_persistent(g, p.variant, NUM_CU, stream);
-        } else {
-            e = launch_tile(g, p.variant, p.ksplit, ws, stream);
-            if (e == hipSuccess && p.ksplit > 1)
-                e = launch_splitk_reduce(g, p.ksplit, ws, stream);
-        }
-        snprintf(t_name_buf, sizeof(t_name_buf), "%s_k%d%s", tile_variant_name(p.variant), p.ksplit,
-                 p.persistent ? "_persistent" : "");
-        t_last_kernel = t_name_buf;
-        break;
-    }
-    }
-    return (int)e;
+    plan_name(p, t_name_buf, sizeof(t_name_buf));
+    t_last_kernel = t_name_buf;
+    return rc;
 }
 
 }  // namespace
@@ -394,13 +489,7 @@ int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap)
     Plan p = make_plan(g, g_selected.load());
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
-    if (p.family == FP8GEMM_KERNEL_SCALAR)
-        snprintf(name, cap, "scalar");
-    else if (p.family == FP8GEMM_KERNEL_SKINNY)
-        snprintf(name, cap, "skinny_k%d", p.ksplit);
-    else
-        snprintf(name, cap, "%s_k%d%s", tile_variant_name(p.variant), p.ksplit,
-                 p.persistent ? "_persistent" : "");
+    plan_name(p, name, cap);
     return FP8GEMM_OK;
 }
 
@@ -413,7 +502,14 @@ size_t fp8_block_gemm_workspace_bytes(int m, int n, int k)
     GemmArgs g{reinterpret_cast<const uint8_t*>(uintptr_t(4096)), reinterpret_cast<const uint8_t*>(uintptr_t(4096)),
                nullptr, nullptr, reinterpret_cast<uint16_t*>(uintptr_t(4096)), m, n, k};
     const Plan p = make_plan(g, g_selected.load());
-    return p.family < 0 ? 0 : plan_workspace_bytes(g, p);
+    if (p.family < 0)
+        return 0;
+    if (!p.padded)
+        return plan_workspace_bytes(g, p);
+    GemmArgs gp = g;
+    gp.m = (m + 15) & ~15;
+    gp.n = (n + 15) & ~15;
+    return pad_layout(g, plan_workspace_bytes(gp, p), true).total;
 }
 
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)

@@ -54,6 +54,13 @@ bool skinny_supports(const GemmArgs& g);
 int skinny_ksplit(const GemmArgs& g);
 hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s);
 
+// rows of ld_src elements copied into rows of ld_dst >= ld_src elements, the rest zero (dst
+// 16-byte aligned, ld_dst a multiple of 16 bytes); the m x n corner of a bf16 matrix with
+// ld_src elements per row copied into a dense one
+hipError_t launch_pad_bytes(const uint8_t* src, uint8_t* dst, int rows, int ld_src, int ld_dst, hipStream_t s);
+hipError_t launch_pad_floats(const float* src, float* dst, int rows, int ld_src, int ld_dst, hipStream_t s);
+hipError_t launch_crop_bf16(const uint16_t* src, uint16_t* dst, int m, int n, int ld_src, hipStream_t s);
+
 // fp32 -> e4m3fn (check.cu:17-22)
 hipError_t launch_convert(const float* in, uint8_t* out, size_t count, hipStream_t s);
 

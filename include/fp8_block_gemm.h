@@ -58,7 +58,12 @@ extern "C" {
 /* The GEMM on the null stream.  Replaces the reference launch
  * in_smem_kernel<<<grid, block, 0, 0>>>(A, B, As, Bs, C, M, N, K)
  * (/root/reference/check.cu:106-114, kernel mn_large.hip:11 / mn_small.hip:10):
- * same argument order and meaning. */
+ * same argument order and meaning.  Any m, n > 0 and k % 128 == 0.  The MFMA kernels take
+ * m % 16 == 0, n % 16 == 0 and 16-byte aligned a, b, a_scale, c as they are; for anything else
+ * the library copies the operands concerned into zero-padded buffers in its workspace, runs
+ * there and copies c's m x n corner out (plans named "padded_...": four small extra launches,
+ * about 2 bytes of extra traffic per operand byte).  The reference requires M, N % 64 (32) == 0
+ * and reads out of bounds otherwise (mn_large.hip:16). */
 int fp8_block_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                    void* c, int m, int n, int k);
 
@@ -104,7 +109,7 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
                            void* const* c, const int* m, int n, int k, void* stream);
 
 /* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
- * 16-byte aligned operands into name[0..cap), e.g. "tile256x192_k1_persistent", "tile128x128_k3", "skinny_k1", "scalar".
+ * 16-byte aligned operands into name[0..cap), e.g. "tile256x192_k1_persistent", "tile128x128_k3", "skinny_k1", "padded_tile64x64_k1", "scalar".
  * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart
  * in the reference (its choice is made by editing the source, README.md:55). */
 int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap);
@@ -118,11 +123,13 @@ const char* fp8_block_gemm_last_kernel(void);
  * A caller that must not allocate can supply its own, 256-byte aligned, of at least
  * fp8_block_gemm_workspace_bytes(m, n, k) bytes for every shape it will pass: that is what
  * the plan for the shape needs under the kernel selection and forced configuration in force
- * when it is asked (0 when the plan does not split K; ask again after changing either).
+ * when it is asked (0 when the plan neither splits K nor pads; for a padded plan an upper bound that holds for
+ * any operand alignment; ask again after changing either).
  * Passing NULL returns to the library-owned buffer.  There is ONE workspace per process,
  * on the device that was current when it was allocated or supplied: calls that split K
- * (fp8_block_gemm_plan names them "..._kN" with N > 1) must not overlap on different streams,
- * and must run on that device; calls that do not split K never touch it.  The reference has
+ * (fp8_block_gemm_plan names them "..._kN" with N > 1) or run on padded copies ("padded_...")
+ * must not overlap on different streams, and must run on that device; other calls never
+ * touch it.  The reference has
  * no workspace (its kernels do not split K: mn_small.hip:28). */
 size_t fp8_block_gemm_workspace_bytes(int m, int n, int k);
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes);

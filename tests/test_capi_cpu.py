@@ -111,7 +111,10 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(8192, 4608, 7168).startswith("tile")
     assert "_k1" in pkg.plan(8192, 4608, 7168)
     assert pkg.plan(32, 7168, 2048).startswith("skinny")
-    assert pkg.plan(33, 100, 128) == "scalar"            # rows not 16-byte aligned
+    assert pkg.plan(33, 100, 128).startswith("padded_")   # rows not 16-byte aligned: padded copies
+    assert pkg.plan(8191, 4607, 7168) == "padded_" + pkg.plan(8192, 4608, 7168)
+    assert pkg.plan(16777215, 16, 128) == "scalar"         # padding would pass the operand size limit
+    assert pkg.workspace_bytes(33, 100, 128) >= 128 * 48 + 128 * 112 + 48 * 4 + 48 * 112 * 2
     ks = int(pkg.plan(2048, 576, 7168).split("_k")[1])
     assert ks > 1                                          # few tiles, long K: split
     pkg.select(pkg.KERNEL_SCALAR)

@@ -132,12 +132,51 @@ def test_skinny_kernel(pkg, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(33, 100, 128), (17, 129, 256), (100, 100, 384)])
-def test_unaligned_shapes_fall_back_to_the_scalar_kernel(pkg, m, n, k):
+def test_scalar_kernel_takes_unaligned_shapes(pkg, m, n, k):
     a, b, sa, sb = oracle.make_inputs(m, n, k, 5 + m)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
-    got, name = _run(pkg, a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SCALAR)
     assert name == "scalar"
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("m,n,k", [(33, 100, 128), (17, 129, 256), (100, 100, 384), (1, 1, 128), (1, 7, 256),
+                                   (5, 1, 128), (250, 300, 512), (1000, 777, 1024), (33, 4100, 1024),
+                                   (2049, 2049, 256), (17, 129, 8192), (8, 8200, 2048), (4100, 24, 1280),
+                                   (255, 257, 384), (1022, 510, 640), (130, 4607, 256)])
+def test_unaligned_shapes_run_on_padded_copies(pkg, m, n, k):
+    """m or n not a multiple of 16: the MFMA kernels run on zero-padded copies in the workspace
+    and C's m x n corner is copied out"""
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 77 + m)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k)
+    assert name.startswith("padded_"), name
+    _assert_close(got, ref, name)
+    assert pkg.plan(m, n, k) == name
+    assert pkg.workspace_bytes(m, n, k) >= ((m + 15) // 16 * 16) * ((n + 15) // 16 * 16) * 2
+    pkg.release()
+
+
+def test_misaligned_operand_addresses_run_on_padded_copies(pkg):
+    """multiples of 16 everywhere, but a, a_scale and c start 4 or 8 bytes off a 16-byte boundary"""
+    import torch
+    m, n, k = 512, 384, 1024
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 78)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    da = torch.zeros(k * m + 16, dtype=torch.uint8, device="cuda")[8:8 + k * m]
+    da.copy_(torch.from_numpy(a).reshape(-1))
+    dsa = torch.zeros(sa.size + 4, dtype=torch.float32, device="cuda")[1:1 + sa.size]
+    dsa.copy_(torch.from_numpy(sa).reshape(-1))
+    dc = torch.full((m * n + 8,), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)[2:2 + m * n]
+    db, dsb = torch.from_numpy(b).cuda(), torch.from_numpy(sb).cuda()
+    assert da.data_ptr() % 16 == 8 and dsa.data_ptr() % 16 == 4 and dc.data_ptr() % 16 == 4
+    _say(f"[gpu case] misaligned operands m={m} n={n} k={k}")
+    pkg.gemm(da, db, dsa, dsb, dc, m, n, k, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    name = pkg.last_kernel()
+    assert name.startswith("padded_"), name
+    _assert_close(dc.cpu().numpy().view(np.uint16).reshape(m, n), ref, name)
+    pkg.release()
 
 
 # ------------------------------------------------------------------ the five benchmark configurations
