@@ -345,10 +345,10 @@ def main():
                 "ms": round(best * 1e3, 2), "tflops": round(flops / best * 1e-12, 2),
                 "host_bytes_moved": moved, "host_gbs": round(moved / best * 1e-9, 1)}
 
-    def grouped_report(steps, warmup):
+    def grouped_report(steps, warmup, ms=(512, 1024, 768, 1536, 256, 2048, 1024, 1024)):
         """cfg2's problem cut into eight groups of ragged M (an MoE layer's experts): one grouped
         launch against eight launches of fp8_block_gemm_stream, same buffers"""
-        ms = [512, 1024, 768, 1536, 256, 2048, 1024, 1024]
+        ms = list(ms)
         gn, gk = 7168, 2048
         bufs = []
         for g, gm in enumerate(ms):
@@ -416,6 +416,9 @@ def main():
     quantisers = None if args.no_shapes else quantiser_report(max(100, args.steps), args.warmup)
     vendor = None if args.no_shapes else vendor_plain_fp8_gemm_us(max(10, args.steps // 2), args.warmup)
     grouped = None if args.no_shapes else grouped_report(max(30, args.steps), args.warmup)
+    if grouped is not None:   # the same token count with group sizes off the 16-row grid: padded copies
+        grouped["off_grid"] = grouped_report(max(30, args.steps), args.warmup,
+                                             ms=(509, 1027, 771, 1533, 250, 2051, 1023, 1028))
     host_boundary = None if args.no_shapes else host_boundary_report()
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,

@@ -48,8 +48,10 @@ struct PadLayout {
 inline size_t round256(size_t x) { return (x + 255) & ~(size_t)255; }
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; }
 
-// conservative = true: every operand copied (an upper bound that does not depend on addresses)
-PadLayout pad_layout(const GemmArgs& g, size_t partial_bytes, bool conservative)
+// conservative = true: every operand copied (an upper bound that does not depend on addresses).
+// keeps_rows = the kernels of the plan take a leading dimension for a and a_scale apart from m
+// (the tile kernels): c then needs no copy on account of m.
+PadLayout pad_layout(const GemmArgs& g, size_t partial_bytes, bool conservative, bool keeps_rows)
 {
     PadLayout L{};
     L.m16 = (g.m + 15) & ~15;
@@ -58,7 +60,7 @@ PadLayout pad_layout(const GemmArgs& g, size_t partial_bytes, bool conservative)
     L.a = conservative || rm || misaligned16(g.a);
     L.as = conservative || rm || misaligned16(g.a_scale);
     L.b = conservative || rn || misaligned16(g.b);
-    L.c = conservative || rm || rn || misaligned16(g.c);
+    L.c = conservative || (rm && !keeps_rows) || rn || misaligned16(g.c);
     const size_t nkb = (size_t)g.k / 128;
     size_t off = 0;
     L.off_a = off;
@@ -288,9 +290,15 @@ hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, hipStre
 int run_padded(const GemmArgs& g, const Plan& p, hipStream_t stream)
 {
     GemmArgs gp = g;
-    gp.m = (g.m + 15) & ~15;
+    const int m16 = (g.m + 15) & ~15;
+    gp.m = m16;
     gp.n = (g.n + 15) & ~15;
-    const PadLayout L = pad_layout(g, plan_workspace_bytes(gp, p), false);
+    const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK;
+    const PadLayout L = pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows);
+    if (!L.c) {  // c is written in place: its m rows, while a and a_scale have m16 per k-row
+        gp.m = g.m;
+        gp.lda = m16;
+    }
     int err;
     float* ws = get_workspace(L.total, &err);
     if (!ws)
@@ -299,12 +307,12 @@ int run_padded(const GemmArgs& g, const Plan& p, hipStream_t stream)
     const int nkb = g.k / 128;
     hipError_t e = hipSuccess;
     if (L.a) {
-        e = launch_pad_bytes(g.a, base + L.off_a, g.k, g.m, gp.m, stream);
+        e = launch_pad_bytes(g.a, base + L.off_a, g.k, g.m, m16, stream);
         gp.a = base + L.off_a;
     }
     if (e == hipSuccess && L.as) {
         float* as = reinterpret_cast<float*>(base + L.off_as);
-        e = launch_pad_floats(g.a_scale, as, nkb, g.m, gp.m, stream);
+        e = launch_pad_floats(g.a_scale, as, nkb, g.m, m16, stream);
         gp.a_scale = as;
     }
     if (e == hipSuccess && L.b) {
@@ -348,6 +356,105 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
     plan_name(p, t_name_buf, sizeof(t_name_buf));
     t_last_kernel = t_name_buf;
     return rc;
+}
+
+// tile shape for a grouped launch: what the cost model picks for the stacked problem, among the
+// shapes that have a persistent form, without a K split; -1 when none can take the table
+int grouped_variant(const GroupTable& tab, int n, int k)
+{
+    long long m_total = 0;
+    for (int g = 0; g < tab.groups; ++g)
+        m_total += tab.m[g];
+    if (m_total > 0x7FFFFFFFll)
+        return -1;
+    int best_v = -1;
+    double best = 1e300;
+    const int fv = g_force_variant.load();
+    const GemmArgs stacked{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], (int)m_total, n, k};
+    for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
+        if ((fv >= 0 && v != fv) || !tile_grouped_supports(tab, n, k, v))
+            continue;
+        const double cst = tile_cost(stacked, v, 1);
+        if (cst < best) {
+            best = cst;
+            best_v = v;
+        }
+    }
+    return best_v;
+}
+
+// Grouped launch for problems off the 16-byte grid: A and a_scale of every group (B and C too
+// when n or one of their addresses is off the grid) go through padded copies in the workspace,
+// one batched copy launch per kind around one grouped GEMM.  Returns GROUPED_NOT_APPLICABLE when it cannot run
+// (the caller then takes the groups one by one).
+constexpr int GROUPED_NOT_APPLICABLE = -1000;
+int run_grouped_padded(const GroupTable& tab, int n, int k, hipStream_t s)
+{
+    const long long lim = 0x7FFFFFFFll;
+    const int n16 = (n + 15) & ~15;
+    const size_t nkb = (size_t)k / 128;
+    bool pad_b = n16 != n, pad_c = n16 != n;
+    for (int g = 0; g < tab.groups; ++g) {
+        pad_b = pad_b || misaligned16(tab.b[g]);
+        pad_c = pad_c || misaligned16(tab.c[g]);
+    }
+    size_t off_a[GroupTable::MAX_GROUPS], off_as[GroupTable::MAX_GROUPS], off_b[GroupTable::MAX_GROUPS],
+        off_c[GroupTable::MAX_GROUPS];
+    size_t off = 0;
+    for (int g = 0; g < tab.groups; ++g) {
+        const long long m16 = (tab.m[g] + 15) & ~15;
+        if (m16 * k > lim || (long long)n16 * k > lim || m16 * n16 > lim)
+            return GROUPED_NOT_APPLICABLE;
+        off_a[g] = off;
+        off += round256((size_t)k * m16);
+        off_as[g] = off;
+        off += round256(nkb * m16 * sizeof(float));
+        off_b[g] = off;
+        off += pad_b ? round256((size_t)k * n16) : 0;
+        off_c[g] = off;
+        off += pad_c ? round256((size_t)m16 * n16 * 2) : 0;
+    }
+    int err;
+    float* ws = get_workspace(off, &err);
+    if (!ws)
+        return err;
+    uint8_t* base = reinterpret_cast<uint8_t*>(ws);
+    GroupTable pt;
+    RepackTable ta, tas, tb, tc;
+    pt.groups = ta.groups = tas.groups = tb.groups = tc.groups = tab.groups;
+    for (int g = 0; g < tab.groups; ++g) {
+        const int m = tab.m[g], m16 = (m + 15) & ~15;
+        pt.a[g] = base + off_a[g];
+        pt.a_scale[g] = reinterpret_cast<const float*>(base + off_as[g]);
+        pt.b[g] = pad_b ? base + off_b[g] : tab.b[g];
+        pt.b_scale[g] = tab.b_scale[g];
+        // c in place keeps its m rows; a and a_scale have m16 per k-row either way
+        pt.c[g] = pad_c ? reinterpret_cast<uint16_t*>(base + off_c[g]) : tab.c[g];
+        pt.m[g] = pad_c ? m16 : m;
+        pt.lda[g] = m16;
+        ta.src[g] = tab.a[g], ta.dst[g] = base + off_a[g], ta.rows[g] = k, ta.ld_src[g] = m, ta.ld_dst[g] = m16;
+        tas.src[g] = tab.a_scale[g], tas.dst[g] = base + off_as[g], tas.rows[g] = (int)nkb, tas.ld_src[g] = m,
+        tas.ld_dst[g] = m16;
+        tb.src[g] = tab.b[g], tb.dst[g] = base + off_b[g], tb.rows[g] = k, tb.ld_src[g] = n, tb.ld_dst[g] = n16;
+        tc.src[g] = base + off_c[g], tc.dst[g] = tab.c[g], tc.rows[g] = m, tc.ld_src[g] = n16, tc.ld_dst[g] = n;
+    }
+    const int v = grouped_variant(pt, n16, k);
+    if (v < 0)
+        return GROUPED_NOT_APPLICABLE;
+    hipError_t e = launch_pad_bytes_batched(ta, s);
+    if (e == hipSuccess)
+        e = launch_pad_floats_batched(tas, s);
+    if (e == hipSuccess && pad_b)
+        e = launch_pad_bytes_batched(tb, s);
+    if (e == hipSuccess)
+        e = launch_tile_grouped(pt, n16, k, v, NUM_CU, s);
+    if (e == hipSuccess && pad_c)
+        e = launch_crop_bf16_batched(tc, s);
+    if (e == hipSuccess) {
+        snprintf(t_name_buf, sizeof(t_name_buf), "padded_%s_k1_grouped%d", tile_variant_name(v), tab.groups);
+        t_last_kernel = t_name_buf;
+    }
+    return (int)e;
 }
 
 }  // namespace
@@ -432,22 +539,9 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
             tab.b_scale[t] = b_scale[g];
             tab.c[t] = static_cast<uint16_t*>(c[g]);
             tab.m[t] = m[g];
+            tab.lda[t] = m[g];
         }
-        // tile shape: what the cost model picks for the stacked problem, among the shapes that
-        // have a persistent form, without a K split
-        int best_v = -1;
-        double best = 1e300;
-        const int fv = g_force_variant.load();
-        GemmArgs stacked{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], (int)m_total, n, k};
-        for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
-            if ((fv >= 0 && v != fv) || !tile_grouped_supports(tab, n, k, v))
-                continue;
-            const double cst = tile_cost(stacked, v, 1);
-            if (cst < best) {
-                best = cst;
-                best_v = v;
-            }
-        }
+        const int best_v = grouped_variant(tab, n, k);
         if (best_v >= 0) {
             const hipError_t e = launch_tile_grouped(tab, n, k, best_v, NUM_CU, s);
             if (e == hipSuccess) {
@@ -456,6 +550,9 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
             }
             return (int)e;
         }
+        const int rc = run_grouped_padded(tab, n, k, s);
+        if (rc != GROUPED_NOT_APPLICABLE)
+            return rc;
     }
     for (int g = 0; g < groups; ++g) {
         if (m[g] == 0)
@@ -509,7 +606,7 @@ size_t fp8_block_gemm_workspace_bytes(int m, int n, int k)
     GemmArgs gp = g;
     gp.m = (m + 15) & ~15;
     gp.n = (n + 15) & ~15;
-    return pad_layout(g, plan_workspace_bytes(gp, p), true).total;
+    return pad_layout(g, plan_workspace_bytes(gp, p), true, false).total;
 }
 
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)

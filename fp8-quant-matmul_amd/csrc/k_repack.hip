@@ -14,39 +14,32 @@ namespace fp8gemm {
 
 namespace {
 
-// dst[r][0..ld_dst) = src[r][0..ld_src) followed by zeros; ld_dst is a multiple of V elements
-// and dst is 16-byte aligned.  One thread writes one 16-byte piece.
-template <typename T>
-__global__ void __launch_bounds__(256)
-pad_rows_kernel(const T* __restrict__ src, T* __restrict__ dst, int rows, int ld_src, int ld_dst)
+// dst[r][0..ld_dst) = src[r][0..ld_src) followed by zeros; ld_dst is a multiple of 4 floats and
+// dst is 16-byte aligned.  One thread (number idx) writes one 16-byte piece.
+__device__ __forceinline__ void pad_piece_floats(const float* __restrict__ src, float* __restrict__ dst, int rows,
+                                                 int ld_src, int ld_dst, size_t idx)
 {
-    constexpr int V = 16 / (int)sizeof(T);
-    const int chunks = ld_dst / V;
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int chunks = ld_dst / 4;
     if (idx >= (size_t)rows * chunks)
         return;
     const int r = (int)(idx / chunks), ch = (int)(idx - (size_t)r * chunks);
-    union {
-        T v[V];
-        uint4 q;
-    } u;
+    float v[4];
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-        const int col = ch * V + j;
-        u.v[j] = col < ld_src ? src[(size_t)r * ld_src + col] : T(0);
+    for (int j = 0; j < 4; ++j) {
+        const int col = ch * 4 + j;
+        v[j] = col < ld_src ? src[(size_t)r * ld_src + col] : 0.0f;
     }
-    *reinterpret_cast<uint4*>(dst + (size_t)r * ld_dst + (size_t)ch * V) = u.q;
+    *reinterpret_cast<float4*>(dst + (size_t)r * ld_dst + (size_t)ch * 4) = make_float4(v[0], v[1], v[2], v[3]);
 }
 
-// The same for bytes, at dword speed whatever the alignment of a source row: the (up to five)
-// aligned dwords that hold the 16 source bytes are read and shifted into place.  The first and
-// the last dword may reach up to 3 bytes beyond the row: they stay inside the aligned dwords
-// that hold the matrix's first and last byte, so no access leaves its pages.
-__global__ void __launch_bounds__(256)
-pad_rows_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int rows, int ld_src, int ld_dst)
+// The same for bytes (ld_dst a multiple of 16), at dword speed whatever the alignment of a source
+// row: the (up to five) aligned dwords that hold the 16 source bytes are read and shifted into
+// place.  The first and the last dword may reach up to 3 bytes beyond the row: they stay inside
+// the aligned dwords that hold the matrix's first and last byte, so no access leaves its pages.
+__device__ __forceinline__ void pad_piece_bytes(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int rows,
+                                                int ld_src, int ld_dst, size_t idx)
 {
     const int chunks = ld_dst / 16;
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)rows * chunks)
         return;
     const int r = (int)(idx / chunks), ch = (int)(idx - (size_t)r * chunks);
@@ -73,11 +66,10 @@ pad_rows_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst
 // dst[m][n] (dense) = src[m][0..n) of a matrix with ld_src elements per row (a multiple of 8, base
 // 16-byte aligned).  One thread moves 8 elements of a row: one 16-byte load, and one store as
 // wide as the destination's alignment allows.
-__global__ void __launch_bounds__(256)
-crop_rows_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int m, int n, int ld_src)
+__device__ __forceinline__ void crop_piece(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int m, int n,
+                                           int ld_src, size_t idx)
 {
     const int chunks = (n + 7) / 8;
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)m * chunks)
         return;
     const int r = (int)(idx / chunks), ch = (int)(idx - (size_t)r * chunks);
@@ -100,14 +92,67 @@ crop_rows_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, i
     }
 }
 
-template <typename T>
-hipError_t launch_pad_typed(const T* src, T* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
+enum RepackKind { REPACK_PAD_BYTES, REPACK_PAD_FLOATS, REPACK_CROP_BF16 };
+
+template <int KIND>
+__device__ __forceinline__ void repack_piece(const void* src, void* dst, int rows, int ld_src, int ld_dst, size_t idx)
 {
-    const size_t pieces = (size_t)rows * (ld_dst / (16 / (int)sizeof(T)));
+    if (KIND == REPACK_PAD_BYTES)
+        pad_piece_bytes(static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), rows, ld_src, ld_dst, idx);
+    else if (KIND == REPACK_PAD_FLOATS)
+        pad_piece_floats(static_cast<const float*>(src), static_cast<float*>(dst), rows, ld_src, ld_dst, idx);
+    else  // rows = m, ld_dst = n
+        crop_piece(static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), rows, ld_dst, ld_src, idx);
+}
+
+template <int KIND>
+__host__ __device__ inline size_t repack_pieces(int rows, int ld_dst)
+{
+    return (size_t)rows * (KIND == REPACK_PAD_BYTES ? ld_dst / 16 : KIND == REPACK_PAD_FLOATS ? ld_dst / 4
+                                                                                                : (ld_dst + 7) / 8);
+}
+
+template <int KIND>
+__global__ void __launch_bounds__(256)
+repack_kernel(const void* __restrict__ src, void* __restrict__ dst, int rows, int ld_src, int ld_dst)
+{
+    repack_piece<KIND>(src, dst, rows, ld_src, ld_dst, (size_t)blockIdx.x * blockDim.x + threadIdx.x);
+}
+
+// one matrix per blockIdx.y
+template <int KIND>
+__global__ void __launch_bounds__(256) repack_batched_kernel(const RepackTable tab)
+{
+    const int g = blockIdx.y;
+    repack_piece<KIND>(tab.src[g], tab.dst[g], tab.rows[g], tab.ld_src[g], tab.ld_dst[g],
+                       (size_t)blockIdx.x * blockDim.x + threadIdx.x);
+}
+
+template <int KIND>
+hipError_t launch_repack(const void* src, void* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
+{
+    const size_t pieces = repack_pieces<KIND>(rows, ld_dst);
     if (pieces == 0)
         return hipSuccess;
-    hipLaunchKernelGGL((pad_rows_kernel<T>), dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s, src, dst,
+    hipLaunchKernelGGL((repack_kernel<KIND>), dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s, src, dst,
                        rows, ld_src, ld_dst);
+    return hipGetLastError();
+}
+
+template <int KIND>
+hipError_t launch_repack_batched(const RepackTable& tab, hipStream_t s)
+{
+    if (tab.groups < 1 || tab.groups > RepackTable::MAX_GROUPS)
+        return hipErrorInvalidValue;
+    size_t most = 0;
+    for (int g = 0; g < tab.groups; ++g) {
+        const size_t pieces = repack_pieces<KIND>(tab.rows[g], tab.ld_dst[g]);
+        most = pieces > most ? pieces : most;
+    }
+    if (most == 0)
+        return hipSuccess;
+    hipLaunchKernelGGL((repack_batched_kernel<KIND>), dim3((unsigned)((most + 255) / 256), (unsigned)tab.groups),
+                       dim3(256), 0, s, tab);
     return hipGetLastError();
 }
 
@@ -115,25 +160,32 @@ hipError_t launch_pad_typed(const T* src, T* dst, int rows, int ld_src, int ld_d
 
 hipError_t launch_pad_bytes(const uint8_t* src, uint8_t* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
 {
-    const size_t pieces = (size_t)rows * (ld_dst / 16);
-    if (pieces == 0)
-        return hipSuccess;
-    hipLaunchKernelGGL(pad_rows_bytes_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s, src, dst,
-                       rows, ld_src, ld_dst);
-    return hipGetLastError();
+    return launch_repack<REPACK_PAD_BYTES>(src, dst, rows, ld_src, ld_dst, s);
 }
 
 hipError_t launch_pad_floats(const float* src, float* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
 {
-    return launch_pad_typed<float>(src, dst, rows, ld_src, ld_dst, s);
+    return launch_repack<REPACK_PAD_FLOATS>(src, dst, rows, ld_src, ld_dst, s);
 }
 
 hipError_t launch_crop_bf16(const uint16_t* src, uint16_t* dst, int m, int n, int ld_src, hipStream_t s)
 {
-    const size_t count = (size_t)m * ((n + 7) / 8);
-    hipLaunchKernelGGL(crop_rows_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, src, dst, m, n,
-                       ld_src);
-    return hipGetLastError();
+    return launch_repack<REPACK_CROP_BF16>(src, dst, m, ld_src, n, s);
+}
+
+hipError_t launch_pad_bytes_batched(const RepackTable& tab, hipStream_t s)
+{
+    return launch_repack_batched<REPACK_PAD_BYTES>(tab, s);
+}
+
+hipError_t launch_pad_floats_batched(const RepackTable& tab, hipStream_t s)
+{
+    return launch_repack_batched<REPACK_PAD_FLOATS>(tab, s);
+}
+
+hipError_t launch_crop_bf16_batched(const RepackTable& tab, hipStream_t s)
+{
+    return launch_repack_batched<REPACK_CROP_BF16>(tab, s);
 }
 
 }  // namespace fp8gemm

@@ -42,7 +42,7 @@ template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
-                 uint16_t* __restrict__ c, float* __restrict__ partial, int M, int N, int K,
+                 uint16_t* __restrict__ c, float* __restrict__ partial, int M, int lda, int N, int K,
                  int tiles_m, int tiles_n, int kb_per_split)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
@@ -97,7 +97,7 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
         const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
         const int cc = (RSA == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSA>(r & 7);
         const bool ok = (16 * cc < BM) && (m0 + 16 * cc < M);
-        voff_a[q] = ok ? (uint32_t)(r * M + m0 + 16 * cc) : 0x80000000u;
+        voff_a[q] = ok ? (uint32_t)(r * lda + m0 + 16 * cc) : 0x80000000u;
     }
 #pragma unroll
     for (int q = 0; q < S::NVB; ++q) {
@@ -106,8 +106,8 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
         const bool ok = (16 * cc < BN) && (n0 + 16 * cc < N);
         voff_b[q] = ok ? (uint32_t)(r * N + n0 + 16 * cc) : 0x80000000u;
     }
-    const uint32_t a_bytes = (uint32_t)M * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
-    const uint32_t as_bytes = (uint32_t)nkb * (uint32_t)M * 4u;
+    const uint32_t a_bytes = (uint32_t)lda * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
+    const uint32_t as_bytes = (uint32_t)nkb * (uint32_t)lda * 4u;
     const uint32_t voff_s =
         (4 * lane < BM && m0 + 4 * lane < M) ? (uint32_t)((m0 + 4 * lane) * 4) : 0x80000000u;
 
@@ -119,13 +119,13 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
         const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
         if (q < NA) {
             lds_dma16(rsrc_a, voff_a[S::template voff_index<RSA>(q)], stage + (uint32_t)((NA * wave + q) * 1024),
-                      (uint32_t)(kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)M);
+                      (uint32_t)(kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)lda);
         } else if (q < NA + NB) {
             lds_dma16(rsrc_b, voff_b[S::template voff_index<RSB>(q - NA)],
                       stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
                       (uint32_t)(kb * KBLOCK + S::template extra_rows<RSB>(q - NA)) * (uint32_t)N);
         } else if (wave == 0) {
-            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)kb * (uint32_t)M * 4u);
+            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)kb * (uint32_t)lda * 4u);
         }
     };
 
@@ -385,7 +385,7 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
         if (e != hipSuccess)
             return e;
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
-                           g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
+                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split);
     } else {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -393,7 +393,7 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
         if (e != hipSuccess)
             return e;
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
-                           g.c, partial, g.m, g.n, g.k, tiles_m, tiles_n, kb_per_split);
+                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split);
     }
     return hipGetLastError();
 }
@@ -402,8 +402,10 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
 
 bool tile_supports(const GemmArgs& g)
 {
-    // 16-byte copies need every k-row of a, b and a_scale to start 16-byte aligned
-    return g.m % 16 == 0 && g.n % 16 == 0 && (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) &&
+    // 16-byte copies need every k-row of a, b and a_scale to start 16-byte aligned; rows of a
+    // and a_scale beyond m, up to the leading dimension, are read (and must be finite: zeros)
+    return leading_dim(g) % 16 == 0 && leading_dim(g) >= g.m && g.n % 16 == 0 &&
+           (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.b) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.a_scale) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.c) % 16 == 0);

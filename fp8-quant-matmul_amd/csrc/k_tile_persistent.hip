@@ -30,6 +30,7 @@ struct Problem {
     const float* b_scale;
     uint16_t* c;
     int M;
+    int lda;  // elements between consecutive k-rows of a and of a_scale (>= M, a multiple of 16)
 };
 
 // GROUPED = false: one problem (`one`), tiles_m x tiles_n tiles.  GROUPED = true: the problems of
@@ -82,7 +83,7 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
             while (g + 1 < tab->groups && logical >= tab->tile_start[g + 1])
                 ++g;
             logical -= tab->tile_start[g];
-            pr = Problem{tab->a[g], tab->b[g], tab->a_scale[g], tab->b_scale[g], tab->c[g], tab->m[g]};
+            pr = Problem{tab->a[g], tab->b[g], tab->a_scale[g], tab->b_scale[g], tab->c[g], tab->m[g], tab->lda[g]};
             tm = (pr.M + BM - 1) / BM;
         } else {
             pr = one;
@@ -99,12 +100,12 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
     const int sn = (N + KBLOCK - 1) / KBLOCK;
     // buffer resources of the copy stream's current tile (fixed for a single problem)
     v4i rsrc_a, rsrc_b, rsrc_s;
-    int f_M = one.M;  // rows of the problem the copy stream is in
+    int f_lda = one.lda;  // leading dimension of the problem the copy stream is in
     auto set_resources = [&](const Problem& pr) __attribute__((always_inline)) {
-        rsrc_a = make_rsrc_words(pr.a, (uint32_t)pr.M * (uint32_t)K);
+        rsrc_a = make_rsrc_words(pr.a, (uint32_t)pr.lda * (uint32_t)K);
         rsrc_b = make_rsrc_words(pr.b, (uint32_t)N * (uint32_t)K);
-        rsrc_s = make_rsrc_words(pr.a_scale, (uint32_t)nkb * (uint32_t)pr.M * 4u);
-        f_M = pr.M;
+        rsrc_s = make_rsrc_words(pr.a_scale, (uint32_t)nkb * (uint32_t)pr.lda * 4u);
+        f_lda = pr.lda;
     };
 
     // ---- the copy stream: K block f_kb of this workgroup's tile number f_tile is the next one
@@ -118,13 +119,13 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
         tile_origin(j, pr, m0, n0);
         if (GROUPED || j == 0)
             set_resources(pr);
-        const int M = pr.M;
+        const int M = pr.M, lda = pr.lda;
 #pragma unroll
         for (int q = 0; q < S::NVA; ++q) {
             const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
             const int cc = (RSA == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSA>(r & 7);
             const bool ok = (16 * cc < BM) && (m0 + 16 * cc < M);
-            voff_a[q] = ok ? (uint32_t)(r * M + m0 + 16 * cc) : 0x80000000u;
+            voff_a[q] = ok ? (uint32_t)(r * lda + m0 + 16 * cc) : 0x80000000u;
         }
 #pragma unroll
         for (int q = 0; q < S::NVB; ++q) {
@@ -140,13 +141,13 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
         const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
         if (q < NA) {
             lds_dma16(rsrc_a, voff_a[S::template voff_index<RSA>(q)], stage + (uint32_t)((NA * wave + q) * 1024),
-                      (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)f_M);
+                      (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSA>(q)) * (uint32_t)f_lda);
         } else if (q < NA + NB) {
             lds_dma16(rsrc_b, voff_b[S::template voff_index<RSB>(q - NA)],
                       stage + S::MAT_A + (uint32_t)((NB * wave + (q - NA)) * 1024),
                       (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSB>(q - NA)) * (uint32_t)N);
         } else if (wave == 0) {
-            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)f_kb * (uint32_t)f_M * 4u);
+            lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)f_kb * (uint32_t)f_lda * 4u);
         }
     };
     auto fill_advance = [&]() __attribute__((always_inline)) {
@@ -369,9 +370,9 @@ template <int BM, int BN, int WM, int WN, int NS, int PR>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                             const float* __restrict__ a_scale, const float* __restrict__ b_scale,
-                            uint16_t* __restrict__ c, int M, int N, int K, int tiles_m, int tiles_n)
+                            uint16_t* __restrict__ c, int M, int lda, int N, int K, int tiles_m, int tiles_n)
 {
-    const Problem one{a, b, a_scale, b_scale, c, M};
+    const Problem one{a, b, a_scale, b_scale, c, M, lda};
     persistent_body<BM, BN, WM, WN, NS, PR, false>(one, nullptr, N, K, tiles_m, tiles_n);
 }
 
@@ -379,7 +380,7 @@ template <int BM, int BN, int WM, int WN, int NS, int PR>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_grouped_kernel(const GroupTable tab, int N, int K, int tiles_n)
 {
-    const Problem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    const Problem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
     persistent_body<BM, BN, WM, WN, NS, PR, true>(none, &tab, N, K, 0, tiles_n);
 }
 
@@ -395,7 +396,7 @@ hipError_t launch_persistent_variant(const GemmArgs& g, int workgroups, hipStrea
     if (e != hipSuccess)
         return e;
     hipLaunchKernelGGL(kern, dim3(workgroups), dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale,
-                       g.b_scale, g.c, g.m, g.n, g.k, tiles_m, tiles_n);
+                       g.b_scale, g.c, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n);
     return hipGetLastError();
 }
 
@@ -456,7 +457,7 @@ bool tile_grouped_supports(const GroupTable& tab, int n, int k, int variant)
     if (stages == 0 || k / KBLOCK < stages - 1 || tab.groups < 1 || tab.groups > GroupTable::MAX_GROUPS)
         return false;
     for (int g = 0; g < tab.groups; ++g) {
-        const GemmArgs ga{tab.a[g], tab.b[g], tab.a_scale[g], tab.b_scale[g], tab.c[g], tab.m[g], n, k};
+        const GemmArgs ga{tab.a[g], tab.b[g], tab.a_scale[g], tab.b_scale[g], tab.c[g], tab.m[g], n, k, tab.lda[g]};
         if (tab.m[g] <= 0 || !tile_supports(ga))
             return false;
     }

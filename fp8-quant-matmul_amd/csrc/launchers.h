@@ -14,7 +14,11 @@ struct GemmArgs {
     const float* b_scale;
     uint16_t* c;
     int m, n, k;
+    // elements between consecutive k-rows of a and of a_scale; 0 = m (the layout of the ABI).
+    // Only the tile kernels take another value (padded copies whose c keeps m rows).
+    int lda = 0;
 };
+inline int leading_dim(const GemmArgs& g) { return g.lda ? g.lda : g.m; }
 
 // one thread per C element (check.cu:30-49)
 hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);
@@ -42,6 +46,7 @@ struct GroupTable {
     const float* b_scale[MAX_GROUPS];
     uint16_t* c[MAX_GROUPS];
     int m[MAX_GROUPS];
+    int lda[MAX_GROUPS];  // as GemmArgs::lda, but always filled in
     int tile_start[MAX_GROUPS + 1];
     int groups;
 };
@@ -60,6 +65,21 @@ hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s);
 hipError_t launch_pad_bytes(const uint8_t* src, uint8_t* dst, int rows, int ld_src, int ld_dst, hipStream_t s);
 hipError_t launch_pad_floats(const float* src, float* dst, int rows, int ld_src, int ld_dst, hipStream_t s);
 hipError_t launch_crop_bf16(const uint16_t* src, uint16_t* dst, int m, int n, int ld_src, hipStream_t s);
+// the same for several matrices in one launch (the table travels by value in the kernel
+// arguments).  Padding: rows x ld_src -> rows x ld_dst.  Cropping: rows = m, ld_src = elements
+// per source row, ld_dst = n.
+struct RepackTable {
+    static constexpr int MAX_GROUPS = 64;
+    const void* src[MAX_GROUPS];
+    void* dst[MAX_GROUPS];
+    int rows[MAX_GROUPS];
+    int ld_src[MAX_GROUPS];
+    int ld_dst[MAX_GROUPS];
+    int groups;
+};
+hipError_t launch_pad_bytes_batched(const RepackTable& tab, hipStream_t s);
+hipError_t launch_pad_floats_batched(const RepackTable& tab, hipStream_t s);
+hipError_t launch_crop_bf16_batched(const RepackTable& tab, hipStream_t s);
 
 // fp32 -> e4m3fn (check.cu:17-22)
 hipError_t launch_convert(const float* in, uint8_t* out, size_t count, hipStream_t s);

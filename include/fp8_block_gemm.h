@@ -98,10 +98,12 @@ int fp8_block_gemm_set_persistent(int mode);
  * (ragged M, e.g. the experts of one MoE layer), C[g] = A[g] . B[g]^T with the layouts above.
  * a, b, a_scale, b_scale, c and m are HOST arrays of `groups` entries; the pointers they hold
  * are device pointers.  Groups with m[g] == 0 are skipped.  Up to FP8GEMM_MAX_GROUPS problems
- * whose m[g] are multiples of 16 run as ONE launch of the persistent tile kernel (their tiles
- * form one list that 256 workgroups walk through); anything else falls back to one call of
- * fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to what
- * fp8_block_gemm_stream gives for that problem with the same tile shape.  No counterpart in the
+ * run as ONE launch of the persistent tile kernel (their tiles form one list that 256
+ * workgroups walk through): as they are when every m[g] and n are multiples of 16 and the
+ * operands 16-byte aligned, else on zero-padded copies in the workspace made by one batched copy
+ * launch per operand kind ("padded_..._groupedN").  More groups than that fall back to one call
+ * of fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to
+ * what fp8_block_gemm_stream gives for that problem with the same tile shape.  No counterpart in the
  * reference, which launches one problem at a time (/root/reference/check.cu:106-114). */
 #define FP8GEMM_MAX_GROUPS 64
 int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* b,

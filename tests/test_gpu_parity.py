@@ -405,13 +405,43 @@ def test_grouped_gemm_equals_the_problems_one_by_one(pkg, variant, ms, n, k):
         assert np.array_equal(got, single), f"group {g}: grouped launch and single launch differ"
 
 
-def test_grouped_gemm_falls_back_for_unaligned_groups(pkg):
-    ms, n, k = [40, 256, 24], 256, 256       # 40 and 24 rows: not multiples of 16
-    host, dev, outs, name = _grouped_case(pkg, ms, n, k, -1, 8100)
+@pytest.mark.parametrize("ms,n,k", [([40, 256, 24], 256, 256), ([1, 0, 1000, 333, 16], 520, 384),
+                                    ([129] * 20, 100, 512), ([2049, 17], 1544, 1024)])
+def test_grouped_gemm_pads_groups_off_the_16_byte_grid(pkg, ms, n, k):
+    """ragged m (and n): one grouped launch on padded copies, C rows beyond m untouched"""
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    host, dev, outs = [], [], []
+    for g, m in enumerate(ms):
+        mm = max(m, 1)
+        a, b, sa, sb = oracle.make_inputs(mm, n, k, 8100 + 13 * g)
+        host.append((a, b, sa, sb))
+        dev.append(_dev(a, b, sa, sb))
+        outs.append(torch.full((mm + 16, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16))  # 16 guard rows
+    _say(f"[gpu case] grouped, padded ms={ms} n={n} k={k}")
+    pkg.gemm_grouped([d[0] for d in dev], [d[1] for d in dev], [d[2] for d in dev], [d[3] for d in dev],
+                     outs, ms, n, k, st)
+    torch.cuda.synchronize()
+    name = pkg.last_kernel()
+    assert name.startswith("padded_") and name.endswith(f"_grouped{sum(1 for m in ms if m)}"), name
+    for g, m in enumerate(ms):
+        got = outs[g].cpu().numpy().view(np.uint16)
+        assert (got[m:] == 0x7FC1).all(), f"group {g}: rows beyond m written"
+        if m:
+            a, b, sa, sb = host[g]
+            _assert_close(got[:m], oracle.ref_gemm(a, b, sa, sb, m, n, k), f"{name} group {g}")
+    pkg.release()
+
+
+def test_grouped_gemm_takes_more_groups_than_one_launch_holds(pkg):
+    """70 groups (one launch holds 64): the groups run one by one, ragged ones on padded copies"""
+    ms, n, k = [16 + (g % 3) for g in range(70)], 64, 128
+    host, dev, outs, name = _grouped_case(pkg, ms, n, k, -1, 8300)
     assert "_grouped" not in name, name
     for g, m in enumerate(ms):
         a, b, sa, sb = host[g]
         _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
+    pkg.release()
 
 
 def test_seeded_sweep_of_shapes_and_plans(pkg):
