@@ -50,6 +50,9 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
     static_assert(PR % 32 == 0 && BM % PR == 0, "a piece is a whole number of 32-row patches");
     static_assert(PR * CROW <= S::STAGE, "a piece must fit one ring slot");
     constexpr int CPR = BN / 8;               // 16-byte chunks per tile row
+    // fold of a patch column under the next column's MFMAs: pays for the 2 x 3 patches of the
+    // 256 x 192 tile (4 % there), not for the smaller wave tiles (0 to -2 %)
+    constexpr bool PIPELINED_FOLD = MI * NJ >= 6;
     constexpr int CHUNKS = PR * CPR;
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -268,33 +271,83 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
                         ++cq;
                     }
             };
-#pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                const v8i fb0 = read_frag(addr_b[jj] + so, 0, RSB);
-                const v8i fb1 = read_frag(addr_b[jj] + so, 1, RSB);
+            if (PIPELINED_FOLD) {
+                // Column jj's MFMAs write the block sums that column jj-1's fold has just read: the
+                // fold of patch (i, jj-1) sits in program order right before the first MFMA of
+                // patch (i, jj), pinned there (an empty asm statement that both the folded
+                // accumulator and the MFMA's B fragment pass through), so that its 16 FMAs issue
+                // while the MFMAs before it are still in the pipe.  Left alone, the compiler issues
+                // all MFMAs of a K block first and all folds after them, the matrix pipe idle
+                // meanwhile (both waves of a SIMD reach that phase together, after the barrier).
                 v16f blk[MI];
+                float sc_prev[MI];
 #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
-                                                                              0, 0, 0);
-                    copy_slot(PER_MFMA);
+                for (int jj = 0; jj <= NJ; ++jj) {
+                    v8i fb0, fb1;
+                    if (jj < NJ) {
+                        fb0 = read_frag(addr_b[jj] + so, 0, RSB);
+                        fb1 = read_frag(addr_b[jj] + so, 1, RSB);
+                    }
+#pragma unroll
+                    for (int i = 0; i < MI; ++i) {
+                        if (jj > 0) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r)
+                                acc[i][jj - 1][r] = fmaf(sc_prev[i], blk[i][r], acc[i][jj - 1][r]);
+                            if (jj < NJ)
+                                asm volatile("" : "+v"(acc[i][jj - 1]), "+v"(fb0));
+                        }
+                        if (jj < NJ) {
+                            blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0,
+                                                                                      0, 0, 0, 0);
+                            copy_slot(PER_MFMA);
+                        }
+                    }
+                    if (jj < NJ) {
+#pragma unroll
+                        for (int i = 0; i < MI; ++i) {
+                            blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0,
+                                                                                      0, 0, 0, 0);
+                            copy_slot(PER_MFMA);
+                        }
+                        // wave-uniform choice of the b_scale value on the scalar unit (bit select),
+                        // then one product per patch
+                        const float sbj = __uint_as_float((__float_as_uint(sb_hi) & hi_mask[jj]) |
+                                                          (__float_as_uint(sb_lo) & ~hi_mask[jj]));
+#pragma unroll
+                        for (int i = 0; i < MI; ++i)
+                            sc_prev[i] = sa[i] * sbj;
+                    }
                 }
+            } else {
 #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
-                                                                              0, 0, 0);
-                    copy_slot(PER_MFMA);
-                }
+                for (int jj = 0; jj < NJ; ++jj) {
+                    const v8i fb0 = read_frag(addr_b[jj] + so, 0, RSB);
+                    const v8i fb1 = read_frag(addr_b[jj] + so, 1, RSB);
+                    v16f blk[MI];
 #pragma unroll
-                for (int i = 0; i < MI; ++i) {
-                    // wave-uniform choice of the b_scale value on the scalar unit (bit select), then one
-                    // product per patch
-                    const float sbj = __uint_as_float((__float_as_uint(sb_hi) & hi_mask[jj]) |
-                                                      (__float_as_uint(sb_lo) & ~hi_mask[jj]));
-                    const float sc = sa[i] * sbj;
+                    for (int i = 0; i < MI; ++i) {
+                        blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0, fa[i][0], zero16, 0, 0, 0,
+                                                                                  0, 0, 0);
+                        copy_slot(PER_MFMA);
+                    }
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[i][jj][r] = fmaf(sc, blk[i][r], acc[i][jj][r]);
+                    for (int i = 0; i < MI; ++i) {
+                        blk[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1, fa[i][1], blk[i], 0, 0, 0,
+                                                                                  0, 0, 0);
+                        copy_slot(PER_MFMA);
+                    }
+#pragma unroll
+                    for (int i = 0; i < MI; ++i) {
+                        // wave-uniform choice of the b_scale value on the scalar unit (bit select), then one
+                        // product per patch
+                        const float sbj = __uint_as_float((__float_as_uint(sb_hi) & hi_mask[jj]) |
+                                                          (__float_as_uint(sb_lo) & ~hi_mask[jj]));
+                        const float sc = sa[i] * sbj;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            acc[i][jj][r] = fmaf(sc, blk[i][r], acc[i][jj][r]);
+                    }
                 }
             }
             copy_slot(NCOPY);

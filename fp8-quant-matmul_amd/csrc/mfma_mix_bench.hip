@@ -1,9 +1,10 @@
 // What does the MI355X sustain for the instruction mix of the block-scaled GEMM, with no
 // memory stalls at all?  Every wave loops over register-resident random fp8 operands and
-// issues, per v_mfma_f32_32x32x64_f8f6f4: NF independent v_fmac_f32 (the scale fold needs 8)
-// and NR ds_read_b64_tr_b8 (the 64x96 wave tile needs 3.3).  Two waves per SIMD, 256
-// workgroups.  The figures bound what any schedule of that mix can reach on this part.
-// Usage: mfma_mix_bench [iterations]
+// issues, per v_mfma_f32_32x32x64_f8f6f4: NF v_fmac_f32 on the result of an earlier MFMA (the
+// scale fold needs 8) and NR ds_read_b64_tr_b8 (the 64x96 wave tile needs 3.3).  Two waves per
+// SIMD, 256 workgroups, nothing else in the loop: no barrier, no wait on memory, no copy.  The
+// figures bound what any schedule of that mix can reach on this part.
+// Usage: mfma_mix_bench [iterations [constant]]
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -52,7 +53,7 @@ __global__ void __launch_bounds__(512) mix_kernel(const v8i* data, float* out, i
         for (int u = 0; u < 4; ++u) {
             asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0"
                          : "+v"(acc[u])
-                         : "v"(x[u]), "v"(y[(u + it) & 3]));
+                         : "v"(x[u]), "v"(y[u]));  // fixed registers: a run-time index would cost moves
 #pragma unroll
             for (int j = 0; j < NF; ++j)
                 asm volatile("v_fmac_f32 %0, %1, %2"
