@@ -87,22 +87,22 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     const int kb1 = (kb0 + kb_per_split < nkb) ? (kb0 + kb_per_split) : nkb;
 
     // ---- global -> LDS copy plan.  One 16-byte load per lane fills 1 KiB of LDS (LDS address
-    // = base + lane*16): 4 rows of 256 B or 8 rows of 128 B.  Wave w owns instructions
+    // = base + lane*16): 4 rows of 256 B, 8 rows of 128 B or 16 rows of 64 B.  Wave w owns instructions
     // NA*w .. NA*w+NA-1 of the A tile and likewise of B.  A lane writes chunk position p of
     // row r and therefore fetches column chunk p ^ swizzle(r).  Chunks outside the tile or the
     // matrix get an out-of-range offset: the buffer load then writes zeros and reads nothing.
     uint32_t voff_a[S::NVA], voff_b[S::NVB];
 #pragma unroll
     for (int q = 0; q < S::NVA; ++q) {
-        const int r = RSA == 256 ? (NA * wave + q) * 4 + (lane >> 4) : (NA * wave + q) * 8 + (lane >> 3);
-        const int cc = (RSA == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSA>(r & 7);
+        const int r = (NA * wave + q) * (1024 / RSA) + S::template copy_row<RSA>(lane);
+        const int cc = S::template copy_pos<RSA>(lane) ^ row_swizzle<RSA>(r & 7);
         const bool ok = (16 * cc < BM) && (m0 + 16 * cc < M);
         voff_a[q] = ok ? (uint32_t)(r * lda + m0 + 16 * cc) : 0x80000000u;
     }
 #pragma unroll
     for (int q = 0; q < S::NVB; ++q) {
-        const int r = RSB == 256 ? (NB * wave + q) * 4 + (lane >> 4) : (NB * wave + q) * 8 + (lane >> 3);
-        const int cc = (RSB == 256 ? (lane & 15) : (lane & 7)) ^ row_swizzle<RSB>(r & 7);
+        const int r = (NB * wave + q) * (1024 / RSB) + S::template copy_row<RSB>(lane);
+        const int cc = S::template copy_pos<RSB>(lane) ^ row_swizzle<RSB>(r & 7);
         const bool ok = (16 * cc < BN) && (n0 + 16 * cc < N);
         voff_b[q] = ok ? (uint32_t)(r * N + n0 + 16 * cc) : 0x80000000u;
     }

@@ -14,8 +14,8 @@ constexpr int GROUP_M = 8;  // tile rows per L2 locality group
 
 template <int BM, int BN, int WM, int WN, int NS>
 struct TileShape {
-    static constexpr int RSA = BM > 128 ? 256 : 128;  // LDS bytes per k-row of the A tile
-    static constexpr int RSB = BN > 128 ? 256 : 128;
+    static constexpr int RSA = BM > 128 ? 256 : (BM > 64 ? 128 : 64);  // LDS bytes per k-row of the A tile
+    static constexpr int RSB = BN > 128 ? 256 : (BN > 64 ? 128 : 64);
     static constexpr int MAT_A = KBLOCK * RSA;
     static constexpr int MAT_B = KBLOCK * RSB;
     static constexpr int SCALE_OFF = MAT_A + MAT_B;       // BM a_scale floats
@@ -24,15 +24,21 @@ struct TileShape {
     static constexpr int NA = RSA / 64;                   // copy instructions per wave, A tile
     static constexpr int NB = RSB / 64;
     static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only)
-    // A wave's copy instructions of one matrix lie 4 (256-byte rows) or 8 (128-byte rows) k-rows
-    // apart.  Instructions 8 rows apart share the chunk swizzle and hence the per-lane offset:
-    // only NV distinct offsets are kept in registers, the row distance goes into the
-    // instruction's scalar offset.
+    // A wave's copy instructions of one matrix lie 4 (256-byte rows), 8 (128-byte rows) or 16
+    // (64-byte rows) k-rows apart.  Instructions 8 rows apart share the chunk swizzle and hence
+    // the per-lane offset: only NV distinct offsets are kept in registers, the row distance goes
+    // into the instruction's scalar offset.
     static constexpr int NVA = RSA == 256 ? 2 : 1;
     static constexpr int NVB = RSB == 256 ? 2 : 1;
     // instruction q of a matrix with row stride RS: which kept offset, and how many k-rows on top
     template <int RS> static constexpr int voff_index(int q) { return RS == 256 ? (q & 1) : 0; }
-    template <int RS> static constexpr int extra_rows(int q) { return RS == 256 ? (q >> 1) * 8 : q * 8; }
+    template <int RS> static constexpr int extra_rows(int q)
+    {
+        return RS == 256 ? (q >> 1) * 8 : q * (1024 / RS);
+    }
+    // lane of a copy instruction -> k-row within the instruction's 1 KiB and chunk position in it
+    template <int RS> static __device__ __forceinline__ int copy_row(int lane) { return lane / (RS / 16); }
+    template <int RS> static __device__ __forceinline__ int copy_pos(int lane) { return lane % (RS / 16); }
     static_assert(LDS_BYTES <= 160 * 1024, "stages exceed the 160 KiB of LDS");
 };
 
@@ -40,7 +46,7 @@ struct TileShape {
 template <int RS>
 __device__ __forceinline__ int row_swizzle(int r)
 {
-    return RS == 256 ? 2 * (r & 7) : 2 * ((r >> 1) & 3);
+    return RS == 256 ? 2 * (r & 7) : (RS == 128 ? 2 * ((r >> 1) & 3) : 2 * ((r >> 2) & 1));
 }
 
 template <int N>
