@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
                  uint16_t* __restrict__ c, float* __restrict__ partial, int M, int lda, int N, int K,
-                 int tiles_m, int tiles_n, int kb_per_split)
+                 int tiles_m, int tiles_n, int kb_per_split, int group_m)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
     // Eight waves copy; WM x WN of them (all eight, or the first four for the smallest tile)
@@ -68,16 +68,17 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     const bool compute = NCW == 8 || wave < NCW;
 
     // ---- which tile: consecutive workgroup ids land on different XCDs (id % 8), so give
-    // each XCD a contiguous run of tile numbers, and walk tiles in groups of GROUP_M rows
-    // so that the tiles an XCD works on together share A and B panels in its L2.
+    // each XCD a contiguous run of tile numbers, and walk tiles in groups of group_m rows
+    // so that the tiles an XCD works on together share A and B panels in its L2 (the host picks
+    // group_m so that an XCD's co-resident tiles form a block that is about square in bytes).
     const int T = tiles_m * tiles_n;
     const int pid = blockIdx.x;
     const int xcd = pid & 7, q8 = T >> 3, r8 = T & 7;
     const int logical = xcd * q8 + (xcd < r8 ? xcd : r8) + (pid >> 3);
-    const int per_group = GROUP_M * tiles_n;
+    const int per_group = group_m * tiles_n;
     const int group = logical / per_group;
-    const int first_m = group * GROUP_M;
-    const int gsz = (tiles_m - first_m < GROUP_M) ? (tiles_m - first_m) : GROUP_M;
+    const int first_m = group * group_m;
+    const int gsz = (tiles_m - first_m < group_m) ? (tiles_m - first_m) : group_m;
     const int in_group = logical - group * per_group;
     const int m0 = (first_m + in_group % gsz) * BM;
     const int n0 = (in_group / gsz) * BN;
@@ -368,6 +369,57 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restr
     *reinterpret_cast<uint2*>(c + i4) = pk;
 }
 
+// Tile rows per locality group.  The kernel gives XCD x (workgroup id % 8) a contiguous run of the
+// tile order, which walks the tile grid in groups of group_m rows, column by column.  The tiles an
+// XCD works on together (its first 32: one per CU) then touch some rows of A and some of B; the
+// group size that makes the eight XCDs touch the fewest bytes is found by walking the order, and
+// remembered for the last few grids.
+int choose_group_m(int tiles_m, int tiles_n, int bm, int bn)
+{
+    struct Entry { int tm, tn, bm, bn, g; };
+    static thread_local Entry cache[8] = {};
+    static thread_local int next = 0;
+    for (const Entry& e : cache)
+        if (e.tm == tiles_m && e.tn == tiles_n && e.bm == bm && e.bn == bn)
+            return e.g;
+    const int T = tiles_m * tiles_n;
+    int best_g = GROUP_M;
+    long best_cost = -1;
+    for (int gm = 1; gm <= GROUP_M; ++gm) {
+        long cost = 0;
+        for (int xcd = 0; xcd < 8; ++xcd) {
+            const int q8 = T >> 3, r8 = T & 7;
+            const int start = xcd * q8 + (xcd < r8 ? xcd : r8);
+            int len = q8 + (xcd < r8 ? 1 : 0);
+            len = len < 32 ? len : 32;
+            unsigned long long rows[4] = {0, 0, 0, 0}, cols[4] = {0, 0, 0, 0};  // up to 256 tile rows / columns tracked
+            int nrows = 0, ncols = 0;
+            for (int t = start; t < start + len; ++t) {
+                const int per_group = gm * tiles_n, group = t / per_group, first_m = group * gm;
+                const int gsz = tiles_m - first_m < gm ? tiles_m - first_m : gm;
+                const int in_group = t - group * per_group;
+                const int r = (first_m + in_group % gsz) & 255, c = (in_group / gsz) & 255;
+                if (!(rows[r >> 6] >> (r & 63) & 1)) {
+                    rows[r >> 6] |= 1ull << (r & 63);
+                    ++nrows;
+                }
+                if (!(cols[c >> 6] >> (c & 63) & 1)) {
+                    cols[c >> 6] |= 1ull << (c & 63);
+                    ++ncols;
+                }
+            }
+            cost += (long)nrows * bm + (long)ncols * bn;
+        }
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best_g = gm;
+        }
+    }
+    cache[next] = Entry{tiles_m, tiles_n, bm, bn, best_g};
+    next = (next + 1) & 7;
+    return best_g;
+}
+
 template <int BM, int BN, int WM, int WN, int NS>
 hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStream_t s)
 {
@@ -377,6 +429,7 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
     const int nkb = g.k / KBLOCK;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     dim3 grid(tiles_m * tiles_n, ksplit);
+    const int group_m = choose_group_m(tiles_m, tiles_n, BM, BN);
     hipError_t e;
     if (ksplit > 1) {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
@@ -385,7 +438,7 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
         if (e != hipSuccess)
             return e;
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
-                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split);
+                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
     } else {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -393,7 +446,7 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
         if (e != hipSuccess)
             return e;
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
-                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split);
+                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
     }
     return hipGetLastError();
 }
