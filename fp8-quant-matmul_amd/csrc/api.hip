@@ -116,8 +116,9 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit)
 // Shapes whose best measured plan differs from the model's choice: {m, n, k, variant, ksplit}.
 struct TunedShape { int m, n, k, variant, ksplit; };
 constexpr TunedShape kTuned[] = {
-    {1024, 512, 7168, TILE_128x128, 6},
+    {1024, 512, 7168, TILE_64x64, 2},
     {1024, 576, 7168, TILE_128x128, 4},
+    {6144, 3072, 1536, TILE_256x192, 1},
     {8192, 7168, 2048, TILE_256x192, 1},
 };
 

@@ -93,8 +93,8 @@ def test_workspace_contract(pkg):
     assert pkg.workspace_bytes(0, 8, 128) == 0
     assert pkg.workspace_bytes(64, 64, 128) == 0                     # one K block: nothing to split
     assert pkg.workspace_bytes(8192, 4608, 7168) == 0                # plan does not split K
-    assert pkg.plan(1024, 512, 7168) == "tile128x128_k6"
-    assert pkg.workspace_bytes(1024, 512, 7168) == 6 * 1024 * 512 * 4
+    assert pkg.plan(1024, 512, 7168) == "tile64x64_k2"
+    assert pkg.workspace_bytes(1024, 512, 7168) == 2 * 1024 * 512 * 4
     assert L.fp8_block_gemm_force_config(2, 8) == 0                  # follows a forced configuration
     try:
         assert pkg.workspace_bytes(256, 256, 1024) == 8 * 256 * 256 * 4
