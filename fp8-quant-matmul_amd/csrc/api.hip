@@ -127,6 +127,10 @@ void decide_persistent(const GemmArgs& g, Plan& p)
 {
     p.persistent = false;
     const int mode = g_persistent.load();
+    if (p.variant == TILE_256x192_W4) {  // exists in the persistent form only
+        p.persistent = p.ksplit == 1 && tile_persistent_supports(g, p.variant);
+        return;
+    }
     if (mode == 0 || p.ksplit != 1 || !tile_persistent_supports(g, p.variant))
         return;
     int bm, bn;
@@ -186,7 +190,11 @@ Plan make_plan(const GemmArgs& g, int selected)
             continue;
         if (tile_variant_name(v)[4] == '?')
             continue;
+        if (v == TILE_256x192_W4 && fv != v)  // one-wave-per-SIMD form: only when asked for
+            continue;
         for (int ks = 1; ks <= 16 && ks <= nkb; ++ks) {
+            if (v == TILE_256x192_W4 && ks != 1)
+                continue;
             if (fk > 0 && ks != (fk < nkb ? fk : nkb))
                 continue;
             if (selected == FP8GEMM_KERNEL_LARGE && ks != 1)
@@ -206,10 +214,13 @@ Plan make_plan(const GemmArgs& g, int selected)
             }
         }
     }
-    if (best == 1e300)
+    if (best == 1e300) {
         p.family = -1;
-    else
-        decide_persistent(g, p);
+        return p;
+    }
+    decide_persistent(g, p);
+    if (p.variant == TILE_256x192_W4 && !p.persistent)
+        p.family = -1;
     return p;
 }
 

@@ -10,6 +10,9 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v32f __attribute__((ext_vector_type(32)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v32i __attribute__((ext_vector_type(32)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
@@ -63,13 +66,23 @@ __device__ __forceinline__ v4i make_rsrc_words(const void* base, uint32_t bytes)
 // insertion treats every LDS read after a compiler-visible LDS-writing load as dependent on
 // it and would wait for the copy of the NEXT stage before reading the current one.  The
 // caller orders these copies itself (s_waitcnt vmcnt(0) + barrier before the data is read).
-// M0 is a reserved register that the compiler re-materialises before each of its own uses.
+// M0 is a reserved register: the compiler writes it immediately before each of its own uses and
+// keeps no value in it across other code, and clang rejects it in a clobber list for that reason.
 // soffset is a wave-uniform byte offset added to the global address only (not range checked,
 // not part of the LDS address).
 __device__ __forceinline__ void lds_dma16(v4i rsrc, uint32_t voffset, uint32_t lds_addr,
                                           uint32_t soffset = 0)
 {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %3 offen lds"
+                 :
+                 : "v"(voffset), "s"(rsrc), "s"(lds_addr), "s"(soffset)
+                 : "memory");
+}
+
+// The same with 4 bytes per lane: lane l's dword lands at lds_addr + 4*l (256 bytes per wave).
+__device__ __forceinline__ void lds_dma4(v4i rsrc, uint32_t voffset, uint32_t lds_addr, uint32_t soffset = 0)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %3 offen lds"
                  :
                  : "v"(voffset), "s"(rsrc), "s"(lds_addr), "s"(soffset)
                  : "memory");

@@ -22,6 +22,8 @@ namespace fp8gemm {
 
 namespace {
 
+#include "w4_loop.inc"
+
 // One problem of a grouped launch as the kernel sees it.
 struct Problem {
     const uint8_t* a;
@@ -39,8 +41,10 @@ template <int BM, int BN, int WM, int WN, int NS, int PR, bool GROUPED>
 __device__ __forceinline__ void persistent_body(const Problem& one, const GroupTable* tab, int N, int K,
                                                 int tiles_m, int tiles_n)
 {
-    using S = TileShape<BM, BN, WM, WN, NS>;
-    static_assert(WM * WN == 8, "eight waves per workgroup");
+    constexpr int NW = WM * WN;    // waves per workgroup; four = one wave per SIMD (k_block_w4)
+    constexpr int NTH = 64 * NW;
+    using S = TileShape<BM, BN, WM, WN, NS, NW>;
+    static_assert(NW == 8 || NW == 4, "eight or four waves per workgroup");
     static_assert(NS >= 2 && NS <= 4, "two to four LDS stages");
     constexpr int TM = BM / WM, TN = BN / WN;
     constexpr int MI = TM / 32, NJ = TN / 32;
@@ -49,6 +53,9 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
     constexpr int CROW = BN * 2 + 8;          // staging bytes per tile row (conflict-free writes)
     static_assert(PR % 32 == 0 && BM % PR == 0, "a piece is a whole number of 32-row patches");
     static_assert(PR * CROW <= S::STAGE, "a piece must fit one ring slot");
+    // four waves: the finished tile is staged beside the ring, which then never pauses
+    constexpr int STAGING_W4 = NS * S::STAGE;
+    static_assert(NW == 8 || STAGING_W4 + PR * CROW <= 160 * 1024, "ring and staging area exceed the LDS");
     constexpr int CPR = BN / 8;               // 16-byte chunks per tile row
     // fold of a patch column under the next column's MFMAs: pays for the 2 x 3 patches of the
     // 256 x 192 tile (4 % there), not for the smaller wave tiles (0 to -2 %)
@@ -102,18 +109,19 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
     const int nkb = K / KBLOCK;
     const int sn = (N + KBLOCK - 1) / KBLOCK;
     // buffer resources of the copy stream's current tile (fixed for a single problem)
-    v4i rsrc_a, rsrc_b, rsrc_s;
+    v4i rsrc_a, rsrc_b, rsrc_s, rsrc_bs;
     int f_lda = one.lda;  // leading dimension of the problem the copy stream is in
     auto set_resources = [&](const Problem& pr) __attribute__((always_inline)) {
         rsrc_a = make_rsrc_words(pr.a, (uint32_t)pr.lda * (uint32_t)K);
         rsrc_b = make_rsrc_words(pr.b, (uint32_t)N * (uint32_t)K);
         rsrc_s = make_rsrc_words(pr.a_scale, (uint32_t)nkb * (uint32_t)pr.lda * 4u);
+        rsrc_bs = make_rsrc_words(pr.b_scale, (uint32_t)nkb * (uint32_t)sn * 4u);
         f_lda = pr.lda;
     };
 
     // ---- the copy stream: K block f_kb of this workgroup's tile number f_tile is the next one
     // to be copied.  Per-lane offsets (copy plan of k_tile.hip) belong to that tile.
-    uint32_t voff_a[S::NVA], voff_b[S::NVB], voff_s;
+    uint32_t voff_a[S::NVA], voff_b[S::NVB], voff_s, voff_sb = 0x80000000u;
     int f_tile = 0, f_kb = 0;
     int fill_left = n_my * nkb;  // blocks not yet copied
     auto fill_setup = [&](int j) __attribute__((always_inline)) {
@@ -138,6 +146,8 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
             voff_b[q] = ok ? (uint32_t)(r * N + n0 + 16 * cc) : 0x80000000u;
         }
         voff_s = (4 * lane < BM && m0 + 4 * lane < M) ? (uint32_t)((m0 + 4 * lane) * 4) : 0x80000000u;
+        if (NW == 4)  // lanes 0..3 bring b_scale[kb][n0/128 + lane]
+            voff_sb = (lane < 4 && (n0 >> 7) + lane < sn) ? (uint32_t)(((n0 >> 7) + lane) * 4) : 0x80000000u;
     };
     // copy instruction q of the stream's next block into ring slot `slot`
     auto fill_copy = [&](int slot, int q) __attribute__((always_inline)) {
@@ -151,6 +161,8 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
                       (uint32_t)(f_kb * KBLOCK + S::template extra_rows<RSB>(q - NA)) * (uint32_t)N);
         } else if (wave == 0) {
             lds_dma16(rsrc_s, voff_s, stage + S::SCALE_OFF, (uint32_t)f_kb * (uint32_t)f_lda * 4u);
+        } else if (NW == 4 && wave == 1) {
+            lds_dma4(rsrc_bs, voff_sb, stage + S::SB_OFF, (uint32_t)f_kb * (uint32_t)sn * 4u);
         }
     };
     auto fill_advance = [&]() __attribute__((always_inline)) {
@@ -184,6 +196,190 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
         return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
     };
     const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // ---- a finished tile: bf16, in pieces of PR rows through `staging` (LDS bytes that nobody
+    // else touches meanwhile), 16 bytes per lane along whole tile rows.  A lane owns row
+    // m = .. + (lane & 31) and, per patch, four runs of 4 columns: stored straight from the
+    // registers that would be 8-byte pieces of 32 different rows per instruction.
+    // sum(i, jj, r) = running sum r of patch (i, jj)
+    auto store_tile = [&](auto sum, uint32_t staging, int m0, int n0, int M,
+                          uint16_t* __restrict__ c) __attribute__((always_inline)) {
+        // opaque copy of the thread id: keeps the address arithmetic below inside the tile loop
+        // (hoisted, it would sit in registers the K loop needs and be spilled)
+        int tid = (int)threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane_e = tid & 63;
+#pragma unroll
+        for (int p = 0; p < BM / PR; ++p) {
+            if (p > 0)
+                __syncthreads();  // the previous piece has been read out
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int prow = wm * TM + 32 * i;
+                if (prow / PR == p) {
+                    const uint32_t rbase = staging + (uint32_t)((prow - p * PR + (lane_e & 31)) * CROW);
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int col = wn * TN + 32 * jj + 8 * q + 4 * (lane_e >> 5);
+                            v2i pk = {(int)pack_bf16x2(sum(i, jj, 4 * q), sum(i, jj, 4 * q + 1)),
+                                      (int)pack_bf16x2(sum(i, jj, 4 * q + 2), sum(i, jj, 4 * q + 3))};
+                            *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
+                        }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < (CHUNKS + NTH - 1) / NTH; ++it) {
+                const int idx = it * NTH + tid;
+                const int row = idx / CPR, ch = idx - row * CPR;
+                const int mrow = m0 + p * PR + row;
+                const int ncol = n0 + ch * 8;
+                if (idx < CHUNKS && mrow < M && ncol < N) {
+                    const v2i lo = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16);
+                    const v2i hi = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16 + 8);
+                    *reinterpret_cast<v4i*>(c + (size_t)mrow * N + ncol) = (v4i){lo.x, lo.y, hi.x, hi.y};
+                }
+            }
+        }
+    };
+
+    if constexpr (NW == 4) {
+        // ================= one wave per SIMD =================
+        // A wave owns a 128 x 96 patch grid (2.33 transposing reads per MFMA instead of the 3.33 of
+        // a 64 x 96 wave tile) and all 512 registers of its SIMD lane.  Nobody else issues on the
+        // SIMD, so the K blocks run as one assembly loop with every instruction placed by hand
+        // (w4_loop.inc; schedule, register map and wait counts: gen_w4_loop.py).  What that loop
+        // does differently from the eight-wave schedule below:
+        //   * the barrier of a K block sits before its LAST patch column: by then all fragments of
+        //     the block are in registers, so the slot is free for the block after next right away,
+        //     and the fragments of the next block (landed a whole block ago) are read while the
+        //     last column is multiplied -- no MFMA waits for an LDS round trip behind a barrier;
+        //   * the fold of a block's last patch rides on the first MFMAs of the next block;
+        //   * b_scale rides in the stage like a_scale (a scalar load in flight would turn the
+        //     counted LDS waits into full ones);
+        //   * the finished tile is staged beside the two ring slots: the copy stream never pauses.
+        // This part only walks the tiles, keeps the copy stream's bookkeeping and stores the tiles.
+        static_assert(BM == 256 && BN == 192 && WM == 2 && WN == 2 && NS == 2 && !GROUPED,
+                      "the assembly loop is written for this shape");
+        static_assert(S::STAGE == 66816 && NA == 8 && NB == 8, "ring geometry the assembly loop assumes");
+        const uint32_t scale_kind = wave < 2 ? (uint32_t)wave : 2u;
+        const uint32_t lds_wave = lds_base + (uint32_t)(NA * wave * 1024);
+        const uint32_t lds_scale = lds_base + (wave == 0 ? S::SCALE_OFF : S::SB_OFF);
+        const uint32_t vbase_a0 = lds_base + addr_a[0], vbase_a1 = lds_base + addr_a[1];
+        const uint32_t vbase_a2 = lds_base + addr_a[2], vbase_a3 = lds_base + addr_a[3];
+        const uint32_t vbase_b0 = lds_base + addr_b[0], vbase_b1 = lds_base + addr_b[1], vbase_b2 = lds_base + addr_b[2];
+        const uint32_t vaddr_s = lds_base + addr_s;
+
+        v32f sums[6], blk;
+        v32i frag0 = {}, frag1 = {}, frag2 = {};
+        v16i frag3 = {};
+        float scale_carry = 0.f;
+#pragma unroll
+        for (int r = 0; r < 32; ++r)
+            blk[r] = 0.f;
+
+        // once the stream has run dry its copy instructions stay in the loop with offsets outside
+        // their buffers: they fetch nothing and write zeros into the slot nobody reads
+        auto stream_dry = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < S::NVA; ++q)
+                voff_a[q] = 0x80000000u;
+#pragma unroll
+            for (int q = 0; q < S::NVB; ++q)
+                voff_b[q] = 0x80000000u;
+            voff_s = voff_sb = 0x80000000u;
+        };
+        fill_setup(0);
+#pragma unroll
+        for (int q = 0; q < NCOPY; ++q)
+            fill_copy(0, q);
+        fill_advance();
+        if (fill_left > 0) {
+#pragma unroll
+            for (int q = 0; q < NCOPY; ++q)
+                fill_copy(1, q);
+            fill_advance();
+            wait_vmcnt<NCOPY - 1>();  // block 0 landed (waves 0 and 1: and their first copy of block 1)
+        } else {
+            wait_vmcnt<0>();
+        }
+        if (fill_left == 0)
+            stream_dry();
+        __syncthreads();
+        w4_first_reads(frag0, frag1, frag2, frag3, vbase_a0, vbase_a1, vbase_a2, vbase_a3, vbase_b0);
+
+        uint32_t slot_off = 0;  // LDS offset of the ring slot of the block multiplied next
+        for (int j = 0; j < n_my; ++j) {
+            Problem pr;
+            int m0, n0;
+            tile_origin(j, pr, m0, n0);
+            const int n_wave = n0 + wn * TN;
+            // the stage holds b_scale[kb][n0/128 + 0..3]; a wave's n range touches at most two of them
+            const uint32_t lds_sb_lo = lds_base + S::SB_OFF + 4u * (uint32_t)((n_wave >> 7) - (n0 >> 7));
+            const uint32_t lds_sb_hi = lds_base + S::SB_OFF + 4u * (uint32_t)(((n_wave + TN - 1) >> 7) - (n0 >> 7));
+            uint32_t hi_mask[NJ];  // all ones when patch column jj lies in the wave's second b_scale block
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj)
+                hi_mask[jj] = (uint32_t)-(int)(((n_wave + 32 * jj) >> 7) > (n_wave >> 7));
+#pragma unroll
+            for (int t = 0; t < 6; ++t)
+#pragma unroll
+                for (int r = 0; r < 32; ++r)
+                    sums[t][r] = 0.f;
+
+            int kb = 0;
+            while (kb < nkb) {
+                // as many blocks as the copy stream can take without leaving its tile
+                int cnt = nkb - kb;
+                if (fill_left > 0 && nkb - f_kb < cnt)
+                    cnt = nkb - f_kb;
+                uint32_t count = (uint32_t)cnt;
+                const uint32_t str_a = (uint32_t)(KBLOCK * f_lda), str_b = (uint32_t)(KBLOCK * N);
+                const uint32_t str_sc = wave == 0 ? (uint32_t)f_lda * 4u : (uint32_t)sn * 4u;
+                uint32_t off_a = (uint32_t)f_kb * str_a, off_b = (uint32_t)f_kb * str_b, off_sc = (uint32_t)f_kb * str_sc;
+                // wave-uniform operands of the loop must sit in scalar registers
+                auto sgpr = [](uint32_t x) __attribute__((always_inline)) {
+                    return (uint32_t)__builtin_amdgcn_readfirstlane((int)x);
+                };
+                off_a = sgpr(off_a), off_b = sgpr(off_b), off_sc = sgpr(off_sc), count = sgpr(count);
+                slot_off = sgpr(slot_off);
+                w4_k_blocks(sums[0], sums[1], sums[2], sums[3], sums[4], sums[5], blk, frag0, frag1, frag2, frag3,
+                            scale_carry, vbase_a0, vbase_a1, vbase_a2, vbase_a3, vbase_b0, vbase_b1, vbase_b2,
+                            vaddr_s, voff_a[0], voff_a[1], voff_b[0], voff_b[1], wave == 0 ? voff_s : voff_sb,
+                            rsrc_a, rsrc_b, wave == 0 ? rsrc_s : rsrc_bs, off_a, off_b, off_sc, sgpr(str_a),
+                            sgpr(str_b), sgpr(str_sc), sgpr((uint32_t)(8 * f_lda)), sgpr((uint32_t)(8 * N)), slot_off,
+                            sgpr(lds_wave), sgpr(lds_scale), sgpr(scale_kind), sgpr(lds_sb_lo), sgpr(lds_sb_hi),
+                            sgpr(hi_mask[0]), sgpr(hi_mask[1]), sgpr(hi_mask[2]), count);
+                kb += cnt;
+                if (fill_left > 0) {
+                    fill_left -= cnt;
+                    f_kb += cnt;
+                    if (f_kb == nkb) {
+                        f_kb = 0;
+                        ++f_tile;
+                        if (fill_left > 0)
+                            fill_setup(f_tile);
+                        else
+                            stream_dry();
+                    }
+                }
+            }
+            // the last patch's fold, then the tile leaves through the staging area
+            w4_last_fold(sums[5], blk, scale_carry);
+            scale_carry = 0.f;
+#pragma unroll
+            for (int r = 16; r < 32; ++r)
+                blk[r] = 0.f;
+            store_tile([&](int i, int jj, int r) __attribute__((always_inline)) {
+                           const int q = jj * MI + i;
+                           return sums[q / 2][(q % 2) * 16 + r];
+                       },
+                       (uint32_t)STAGING_W4, m0, n0, pr.M, pr.c);
+        }
+        return;
+    }
 
     // ---- fill the ring: the first NS-1 blocks of the stream
     fill_setup(0);
@@ -368,59 +564,20 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
 
         // ---- epilogue: bf16, in pieces of PR rows through the ring slot of the block multiplied
         // last (slot_fill by now; the stream's next copy goes there, but not before the next
-        // K block's barrier), 16 bytes per lane along whole tile rows.  Every copy of the stream
-        // issued so far has to have landed before the first store goes out: the next tile's
-        // first blocks are then known to be there without a wait that would also cover these
-        // stores.
+        // K block's barrier).  Every copy of the stream issued so far has to have landed before
+        // the first store goes out: the next tile's first blocks are then known to be there
+        // without a wait that would also cover these stores.
         wait_vmcnt<0>();
-        const uint32_t staging = (uint32_t)(slot_fill * S::STAGE);
         __syncthreads();  // every wave has finished reading that slot
-        // opaque copy of the thread id: keeps the address arithmetic below inside the tile loop
-        // (hoisted, it would sit in registers the K loop needs and be spilled)
-        int tid = (int)threadIdx.x;
-        asm volatile("" : "+v"(tid));
-        const int lane_e = tid & 63;
-#pragma unroll
-        for (int p = 0; p < BM / PR; ++p) {
-            if (p > 0)
-                __syncthreads();  // the previous piece has been read out
-#pragma unroll
-            for (int i = 0; i < MI; ++i) {
-                const int prow = wm * TM + 32 * i;
-                if (prow / PR == p) {
-                    const uint32_t rbase = staging + (uint32_t)((prow - p * PR + (lane_e & 31)) * CROW);
-#pragma unroll
-                    for (int jj = 0; jj < NJ; ++jj)
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const int col = wn * TN + 32 * jj + 8 * q + 4 * (lane_e >> 5);
-                            v2i pk = {(int)pack_bf16x2(acc[i][jj][4 * q], acc[i][jj][4 * q + 1]),
-                                      (int)pack_bf16x2(acc[i][jj][4 * q + 2], acc[i][jj][4 * q + 3])};
-                            *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
-                        }
-                }
-            }
-            __syncthreads();
-#pragma unroll
-            for (int it = 0; it < (CHUNKS + NTHREADS - 1) / NTHREADS; ++it) {
-                const int idx = it * NTHREADS + tid;
-                const int row = idx / CPR, ch = idx - row * CPR;
-                const int mrow = m0 + p * PR + row;
-                const int ncol = n0 + ch * 8;
-                if (idx < CHUNKS && mrow < M && ncol < N) {
-                    const v2i lo = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16);
-                    const v2i hi = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16 + 8);
-                    *reinterpret_cast<v4i*>(c + (size_t)mrow * N + ncol) = (v4i){lo.x, lo.y, hi.x, hi.y};
-                }
-            }
-        }
+        store_tile([&](int i, int jj, int r) __attribute__((always_inline)) { return acc[i][jj][r]; },
+                   (uint32_t)(slot_fill * S::STAGE), m0, n0, M, c);
         // the next tile's first K block begins with a barrier: the slot is not written again
         // before every lane has read its chunks of the last piece
     }
 }
 
 template <int BM, int BN, int WM, int WN, int NS, int PR>
-__global__ void __launch_bounds__(NTHREADS)
+__global__ void __launch_bounds__(64 * WM * WN)
 tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                             const float* __restrict__ a_scale, const float* __restrict__ b_scale,
                             uint16_t* __restrict__ c, int M, int lda, int N, int K, int tiles_m, int tiles_n)
@@ -430,7 +587,7 @@ tile_gemm_persistent_kernel(const uint8_t* __restrict__ a, const uint8_t* __rest
 }
 
 template <int BM, int BN, int WM, int WN, int NS, int PR>
-__global__ void __launch_bounds__(NTHREADS)
+__global__ void __launch_bounds__(64 * WM * WN)
 tile_gemm_grouped_kernel(const GroupTable tab, int N, int K, int tiles_n)
 {
     const Problem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
@@ -440,15 +597,16 @@ tile_gemm_grouped_kernel(const GroupTable tab, int N, int K, int tiles_n)
 template <int BM, int BN, int WM, int WN, int NS, int PR>
 hipError_t launch_persistent_variant(const GemmArgs& g, int workgroups, hipStream_t s)
 {
-    using S = TileShape<BM, BN, WM, WN, NS>;
-    constexpr int LDS_TOTAL = S::LDS_BYTES;
+    using S = TileShape<BM, BN, WM, WN, NS, WM * WN>;
+    // four waves stage the finished tile beside the ring
+    constexpr int LDS_TOTAL = S::LDS_BYTES + (WM * WN == 4 ? PR * (BN * 2 + 8) : 0);
     const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     auto kern = tile_gemm_persistent_kernel<BM, BN, WM, WN, NS, PR>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
     if (e != hipSuccess)
         return e;
-    hipLaunchKernelGGL(kern, dim3(workgroups), dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale,
+    hipLaunchKernelGGL(kern, dim3(workgroups), dim3(64 * WM * WN), LDS_TOTAL, s, g.a, g.b, g.a_scale,
                        g.b_scale, g.c, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n);
     return hipGetLastError();
 }
@@ -478,6 +636,7 @@ int persistent_stages(int variant)
     case TILE_256x128: return 3;
     case TILE_128x192: return 3;
     case TILE_128x128: return 4;
+    case TILE_256x192_W4: return 2;
     default: return 0;
     }
 }
@@ -499,6 +658,7 @@ hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups
     case TILE_256x128: return launch_persistent_variant<256, 128, 4, 2, 3, 128>(g, workgroups, s);
     case TILE_128x192: return launch_persistent_variant<128, 192, 4, 2, 3, 128>(g, workgroups, s);
     case TILE_128x128: return launch_persistent_variant<128, 128, 2, 4, 4, 128>(g, workgroups, s);
+    case TILE_256x192_W4: return launch_persistent_variant<256, 192, 2, 2, 2, 64>(g, workgroups, s);
     default: return hipErrorInvalidValue;
     }
 }

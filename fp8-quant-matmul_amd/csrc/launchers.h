@@ -27,7 +27,7 @@ hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);
 // partial sums to `partial` ([ksplit][m][n]) instead of c and must be followed by
 // launch_splitk_reduce.
 enum TileVariant { TILE_256x192 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_128x192 = 3,
-                   TILE_64x64 = 4, TILE_VARIANT_COUNT };
+                   TILE_64x64 = 4, TILE_256x192_W4 = 5, TILE_VARIANT_COUNT };
 bool tile_supports(const GemmArgs& g);
 const char* tile_variant_name(int variant);
 void tile_variant_dims(int variant, int* bm, int* bn);

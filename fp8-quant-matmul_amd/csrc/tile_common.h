@@ -12,18 +12,24 @@ namespace {
 constexpr int NTHREADS = 512;
 constexpr int GROUP_M = 8;  // tile rows per L2 locality group
 
-template <int BM, int BN, int WM, int WN, int NS>
+// NW = waves of the workgroup (all of them copy): eight, or four for the kernels that run one wave
+// per SIMD with twice the registers.
+template <int BM, int BN, int WM, int WN, int NS, int NW = 8>
 struct TileShape {
     static constexpr int RSA = BM > 128 ? 256 : (BM > 64 ? 128 : 64);  // LDS bytes per k-row of the A tile
     static constexpr int RSB = BN > 128 ? 256 : (BN > 64 ? 128 : 64);
     static constexpr int MAT_A = KBLOCK * RSA;
     static constexpr int MAT_B = KBLOCK * RSB;
     static constexpr int SCALE_OFF = MAT_A + MAT_B;       // BM a_scale floats
-    static constexpr int STAGE = MAT_A + MAT_B + 1024;
+    static constexpr int SB_OFF = SCALE_OFF + 1024;       // four waves: 64 dwords, the first four = b_scale
+    static constexpr int STAGE = MAT_A + MAT_B + 1024 + (NW == 4 ? 256 : 0);
     static constexpr int LDS_BYTES = NS * STAGE;
-    static constexpr int NA = RSA / 64;                   // copy instructions per wave, A tile
-    static constexpr int NB = RSB / 64;
-    static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only)
+    static constexpr int NA = RSA / (8 * NW);             // copy instructions per wave, A tile
+    static constexpr int NB = RSB / (8 * NW);
+    static constexpr int NCOPY = NA + NB + 1;             // + the a_scale slice (wave 0 only; four
+                                                          // waves: wave 1 brings b_scale as well)
+    static_assert(NW == 4 || NW == 8, "four or eight waves");
+    static_assert(NA * 8 * NW == RSA && NB * 8 * NW == RSB, "whole copy instructions per wave");
     // A wave's copy instructions of one matrix lie 4 (256-byte rows), 8 (128-byte rows) or 16
     // (64-byte rows) k-rows apart.  Instructions 8 rows apart share the chunk swizzle and hence
     // the per-lane offset: only NV distinct offsets are kept in registers, the row distance goes

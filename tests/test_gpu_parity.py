@@ -109,6 +109,28 @@ def test_tile_kernel_persistent(pkg, variant, m, n, k):
     assert np.array_equal(got, plain), "persistent and plain tile kernels fold the same sums in the same order"
 
 
+# one-wave-per-SIMD form of the 256 x 192 tile (variant 5, persistent only; its K loop is an assembly
+# loop): one tile, fewer tiles than workgroups, several tiles per workgroup, one and two K blocks
+# (the copy stream changes tile in every call of the loop), ragged edges in both directions, and a
+# column count that makes a wave's 96 columns straddle two b_scale blocks in every alignment
+W4_SHAPES = [(256, 192, 128), (512, 384, 256), (1040, 1232, 384), (4096, 3456, 512), (4112, 3472, 128),
+             (2048, 2304, 1024), (8192, 4608, 896), (4400, 3280, 256)]
+
+
+@pytest.mark.parametrize("m,n,k", W4_SHAPES)
+def test_tile_kernel_one_wave_per_simd(pkg, m, n, k):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 5 * m + n + k, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=5)
+    assert name == "tile256x192w4_k1_persistent", name
+    _assert_close(got, ref, name)
+    plain, name0 = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=0, persistent=0)
+    assert name0 == "tile256x192_k1", name0
+    assert np.array_equal(got, plain), "both forms fold the same block sums in the same order"
+    again, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=5)
+    assert np.array_equal(got, again), "run-to-run reproducible"
+
+
 @pytest.mark.parametrize("variant,ksplit,m,n,k", [(2, 2, 256, 256, 512), (2, 4, 512, 512, 1024),
                                                    (1, 3, 272, 576, 896), (0, 8, 256, 576, 2048),
                                                    (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048), (3, 5, 384, 576, 1280),
