@@ -16,6 +16,14 @@ KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5
 DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH = 0, 1, 2
 
 
+class Options(C.Structure):
+    """fp8gemm_options of the header: per-call kernel choice for gemm_ex"""
+    _fields_ = [("kernel", C.c_int), ("tile_variant", C.c_int), ("ksplit", C.c_int), ("persistent", C.c_int)]
+
+    def __init__(self, kernel=KERNEL_AUTO, tile_variant=-1, ksplit=0, persistent=-1):
+        super().__init__(kernel, tile_variant, ksplit, persistent)
+
+
 class Fp8GemmError(RuntimeError):
     def __init__(self, code, where):
         self.code = code
@@ -54,6 +62,14 @@ def lib():
     L.fp8_block_gemm.argtypes = [vp, vp, fp, fp, vp, i, i, i]
     L.fp8_block_gemm_stream.restype = i
     L.fp8_block_gemm_stream.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
+    L.fp8_block_gemm_ex.restype = i
+    L.fp8_block_gemm_ex.argtypes = [vp, vp, fp, fp, vp, i, i, i, C.POINTER(Options), vp, sz, vp]
+    L.fp8_block_gemm_ws.restype = i
+    L.fp8_block_gemm_ws.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp, sz, vp]
+    L.fp8_block_gemm_workspace_bytes_ex.restype = sz
+    L.fp8_block_gemm_workspace_bytes_ex.argtypes = [i, i, i, C.POINTER(Options), i]
+    L.fp8_block_gemm_grouped_workspace_bytes.restype = sz
+    L.fp8_block_gemm_grouped_workspace_bytes.argtypes = [i, C.POINTER(C.c_int), i, i]
     L.fp8_block_gemm_scalar.restype = i
     L.fp8_block_gemm_scalar.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
     L.fp8_block_gemm_select.restype = i
@@ -117,6 +133,25 @@ def gemm(a, b, a_scale, b_scale, c, m, n, k, stream=None):
         rc = L.fp8_block_gemm_stream(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k,
                                      stream)
     _check(rc, "fp8_block_gemm")
+
+
+def gemm_ex(a, b, a_scale, b_scale, c, m, n, k, options=None, workspace=None, workspace_bytes=0, stream=None):
+    """Per-call form: `options` (Options or None = automatic), `workspace` (device tensor / pointer or
+    None) of `workspace_bytes`.  Allocates nothing, reads no process-wide switch."""
+    opt = C.byref(options) if options is not None else None
+    rc = lib().fp8_block_gemm_ex(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k, opt,
+                                 _ptr(workspace), workspace_bytes, stream)
+    _check(rc, "fp8_block_gemm_ex")
+
+
+def workspace_bytes_ex(m, n, k, options=None, any_alignment=False):
+    opt = C.byref(options) if options is not None else None
+    return int(lib().fp8_block_gemm_workspace_bytes_ex(m, n, k, opt, 1 if any_alignment else 0))
+
+
+def grouped_workspace_bytes(m, n, k):
+    ms = (C.c_int * len(m))(*[int(v) for v in m])
+    return int(lib().fp8_block_gemm_grouped_workspace_bytes(len(m), ms, n, k))
 
 
 def gemm_scalar(a, b, a_scale, b_scale, c, m, n, k, stream=None):

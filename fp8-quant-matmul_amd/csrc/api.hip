@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
+#include <vector>
 
 using namespace fp8gemm;
 
@@ -16,6 +17,8 @@ namespace {
 
 constexpr int NUM_CU = 256;
 
+// Process-wide defaults, set by fp8_block_gemm_select / _force_config / _set_persistent and read by
+// the entry points without an options argument.  The _ex / _ws entry points read none of this.
 std::atomic<int> g_selected{FP8GEMM_KERNEL_AUTO};
 std::atomic<int> g_force_variant{-1};
 std::atomic<int> g_force_ksplit{0};
@@ -23,9 +26,28 @@ std::atomic<int> g_persistent{-1};  // -1 = when tiles outnumber the CUs, 0 = ne
 thread_local const char* t_last_kernel = "none";
 thread_local char t_name_buf[64];
 
+// what decides a plan besides the shape
+struct Config {
+    int selected;       // FP8GEMM_KERNEL_*
+    int force_variant;  // tile shape, -1 = cost model
+    int force_ksplit;   // 0 = cost model
+    int persistent;     // -1 / 0 / 1 as above
+};
+Config global_config() { return Config{g_selected.load(), g_force_variant.load(), g_force_ksplit.load(), g_persistent.load()}; }
+constexpr int MAX_KSPLIT = 16;
+
+// device memory a call may use beyond its operands: fp32 partial sums of plans that split K, padded
+// copies of operands off the 16-byte grid
+struct Workspace {
+    float* ptr;
+    size_t bytes;
+};
+
 std::mutex g_ws_mutex;
 float* g_ws_own = nullptr;       // library-owned workspace
 size_t g_ws_own_bytes = 0;
+std::vector<void*> g_ws_retired; // outgrown library-owned buffers: kernels in flight and captured graphs may
+                                 // still use them, so they live until fp8_block_gemm_release()
 float* g_ws_user = nullptr;      // caller-supplied workspace
 size_t g_ws_user_bytes = 0;
 
@@ -123,10 +145,10 @@ constexpr TunedShape kTuned[] = {
 };
 
 // A persistent launch pays off when a CU gets more than one tile.
-void decide_persistent(const GemmArgs& g, Plan& p)
+void decide_persistent(const GemmArgs& g, Plan& p, const Config& cfg)
 {
     p.persistent = false;
-    const int mode = g_persistent.load();
+    const int mode = cfg.persistent;
     if (p.variant == TILE_256x192_W4) {  // exists in the persistent form only
         p.persistent = p.ksplit == 1 && tile_persistent_supports(g, p.variant);
         return;
@@ -139,8 +161,9 @@ void decide_persistent(const GemmArgs& g, Plan& p)
     p.persistent = mode == 1 || tiles > NUM_CU;
 }
 
-Plan make_plan(const GemmArgs& g, int selected)
+Plan make_plan(const GemmArgs& g, const Config& cfg)
 {
+    const int selected = cfg.selected;
     Plan p{FP8GEMM_KERNEL_SCALAR, 0, 1};
     if (selected == FP8GEMM_KERNEL_SCALAR)
         return p;
@@ -169,11 +192,11 @@ Plan make_plan(const GemmArgs& g, int selected)
         const uint8_t* const al8 = reinterpret_cast<const uint8_t*>(uintptr_t(4096));
         GemmArgs gp{al8, al8, reinterpret_cast<const float*>(uintptr_t(4096)), g.b_scale,
                     reinterpret_cast<uint16_t*>(uintptr_t(4096)), (int)m16, (int)n16, g.k};
-        p = make_plan(gp, selected);
+        p = make_plan(gp, cfg);
         p.padded = p.family != FP8GEMM_KERNEL_SCALAR && p.family >= 0;
         return p;
     }
-    const int fv = g_force_variant.load(), fk = g_force_ksplit.load();
+    const int fv = cfg.force_variant, fk = cfg.force_ksplit;
     const int nkb = g.k / 128;
     if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0)
         for (const TunedShape& t : kTuned)
@@ -181,7 +204,7 @@ Plan make_plan(const GemmArgs& g, int selected)
                 p.family = t.ksplit > 1 ? FP8GEMM_KERNEL_SPLITK : FP8GEMM_KERNEL_LARGE;
                 p.variant = t.variant;
                 p.ksplit = t.ksplit;
-                decide_persistent(g, p);
+                decide_persistent(g, p, cfg);
                 return p;
             }
     double best = 1e300;
@@ -192,7 +215,7 @@ Plan make_plan(const GemmArgs& g, int selected)
             continue;
         if (v == TILE_256x192_W4 && fv != v)  // one-wave-per-SIMD form: only when asked for
             continue;
-        for (int ks = 1; ks <= 16 && ks <= nkb; ++ks) {
+        for (int ks = 1; ks <= MAX_KSPLIT && ks <= nkb; ++ks) {
             if (v == TILE_256x192_W4 && ks != 1)
                 continue;
             if (fk > 0 && ks != (fk < nkb ? fk : nkb))
@@ -218,46 +241,44 @@ Plan make_plan(const GemmArgs& g, int selected)
         p.family = -1;
         return p;
     }
-    decide_persistent(g, p);
+    decide_persistent(g, p, cfg);
     if (p.variant == TILE_256x192_W4 && !p.persistent)
         p.family = -1;
     return p;
 }
 
-// fp32 partial buffer of at least `bytes`, or nullptr with *err set
-float* get_workspace(size_t bytes, int* err)
+// The process-wide workspace for a call on `stream` that needs `bytes`: the caller-supplied one, else
+// the library-owned one, grown on demand.  Growing allocates, which a stream under capture does not
+// allow (and which would leave the graph with a buffer it was not recorded with): such a call gets
+// FP8GEMM_E_WORKSPACE and the capture stays valid.  Nothing here waits for the device: an outgrown
+// buffer is retired, not freed.
+int acquire_workspace(size_t bytes, hipStream_t stream, Workspace* out)
 {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    *err = FP8GEMM_OK;
     if (g_ws_user) {
-        if (g_ws_user_bytes < bytes) {
-            *err = FP8GEMM_E_WORKSPACE;
-            return nullptr;
-        }
-        return g_ws_user;
+        if (g_ws_user_bytes < bytes)
+            return FP8GEMM_E_WORKSPACE;
+        *out = Workspace{g_ws_user, g_ws_user_bytes};
+        return FP8GEMM_OK;
     }
     if (g_ws_own_bytes < bytes) {
-        if (g_ws_own) {
-            // kernels of earlier calls may still read the old buffer
-            hipError_t e = hipDeviceSynchronize();
-            if (e != hipSuccess) {
-                *err = (int)e;
-                return nullptr;
-            }
-            (void)hipFree(g_ws_own);
-            g_ws_own = nullptr;
-            g_ws_own_bytes = 0;
-        }
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        hipError_t e = hipStreamIsCapturing(stream, &status);
+        if (e != hipSuccess)
+            return (int)e;
+        if (status != hipStreamCaptureStatusNone)
+            return FP8GEMM_E_WORKSPACE;
         void* p = nullptr;
-        hipError_t e = hipMalloc(&p, bytes);
-        if (e != hipSuccess) {
-            *err = (int)e;
-            return nullptr;
-        }
+        e = hipMalloc(&p, bytes);
+        if (e != hipSuccess)
+            return (int)e;
+        if (g_ws_own)
+            g_ws_retired.push_back(g_ws_own);
         g_ws_own = static_cast<float*>(p);
         g_ws_own_bytes = bytes;
     }
-    return g_ws_own;
+    *out = Workspace{g_ws_own, g_ws_own_bytes};
+    return FP8GEMM_OK;
 }
 
 size_t plan_workspace_bytes(const GemmArgs& g, const Plan& p)
@@ -299,7 +320,17 @@ hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, hipStre
 }
 
 // pad what needs padding into the workspace, run the plan there, copy C's corner out
-int run_padded(const GemmArgs& g, const Plan& p, hipStream_t stream)
+// bytes run_padded needs for this call (depends on which operands are off the grid)
+size_t padded_bytes(const GemmArgs& g, const Plan& p)
+{
+    GemmArgs gp = g;
+    gp.m = (g.m + 15) & ~15;
+    gp.n = (g.n + 15) & ~15;
+    const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK;
+    return pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows).total;
+}
+
+int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t stream)
 {
     GemmArgs gp = g;
     const int m16 = (g.m + 15) & ~15;
@@ -311,11 +342,9 @@ int run_padded(const GemmArgs& g, const Plan& p, hipStream_t stream)
         gp.m = g.m;
         gp.lda = m16;
     }
-    int err;
-    float* ws = get_workspace(L.total, &err);
-    if (!ws)
-        return err;
-    uint8_t* base = reinterpret_cast<uint8_t*>(ws);
+    if (!w.ptr || w.bytes < L.total)
+        return FP8GEMM_E_WORKSPACE;
+    uint8_t* base = reinterpret_cast<uint8_t*>(w.ptr);
     const int nkb = g.k / 128;
     hipError_t e = hipSuccess;
     if (L.a) {
@@ -340,33 +369,38 @@ int run_padded(const GemmArgs& g, const Plan& p, hipStream_t stream)
     return (int)e;
 }
 
+// One GEMM.  explicit_ws = the caller's per-call workspace (its bytes may be 0 / its pointer NULL when the
+// plan needs none); nullptr = the process-wide workspace.
 int run(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k,
-        hipStream_t stream, int selected)
+        hipStream_t stream, const Config& cfg, const Workspace* explicit_ws)
 {
     int v = validate(a, b, as, bs, c, m, n, k);
     if (v != FP8GEMM_OK)
         return v;
     GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), as, bs,
                static_cast<uint16_t*>(c), m, n, k};
-    const Plan p = make_plan(g, selected);
+    const Plan p = make_plan(g, cfg);
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
-    int rc;
-    if (p.padded) {
-        rc = run_padded(g, p, stream);
-    } else {
-        float* ws = nullptr;
-        const size_t need = plan_workspace_bytes(g, p);
-        if (need) {
-            int err;
-            ws = get_workspace(need, &err);
-            if (!ws)
-                return err;
+    const size_t need = p.padded ? padded_bytes(g, p) : plan_workspace_bytes(g, p);
+    Workspace w{nullptr, 0};
+    if (need) {
+        if (explicit_ws) {
+            if (!explicit_ws->ptr || explicit_ws->bytes < need ||
+                (reinterpret_cast<uintptr_t>(explicit_ws->ptr) % 256) != 0)
+                return FP8GEMM_E_WORKSPACE;
+            w = *explicit_ws;
+        } else {
+            const int rc = acquire_workspace(need, stream, &w);
+            if (rc != FP8GEMM_OK)
+                return rc;
         }
-        rc = (int)launch_plan(g, p, ws, stream);
     }
-    plan_name(p, t_name_buf, sizeof(t_name_buf));
-    t_last_kernel = t_name_buf;
+    const int rc = p.padded ? run_padded(g, p, w, stream) : (int)launch_plan(g, p, w.ptr, stream);
+    if (rc == FP8GEMM_OK) {
+        plan_name(p, t_name_buf, sizeof(t_name_buf));
+        t_last_kernel = t_name_buf;
+    }
     return rc;
 }
 
@@ -426,11 +460,13 @@ int run_grouped_padded(const GroupTable& tab, int n, int k, hipStream_t s)
         off_c[g] = off;
         off += pad_c ? round256((size_t)m16 * n16 * 2) : 0;
     }
-    int err;
-    float* ws = get_workspace(off, &err);
-    if (!ws)
-        return err;
-    uint8_t* base = reinterpret_cast<uint8_t*>(ws);
+    Workspace w{nullptr, 0};
+    const int wrc = acquire_workspace(off, s, &w);
+    if (wrc == FP8GEMM_E_WORKSPACE)
+        return GROUPED_NOT_APPLICABLE;  // a caller-supplied workspace sized for single problems: one by one
+    if (wrc != FP8GEMM_OK)
+        return wrc;
+    uint8_t* base = reinterpret_cast<uint8_t*>(w.ptr);
     GroupTable pt;
     RepackTable ta, tas, tb, tc;
     pt.groups = ta.groups = tas.groups = tb.groups = tc.groups = tab.groups;
@@ -469,6 +505,50 @@ int run_grouped_padded(const GroupTable& tab, int n, int k, hipStream_t s)
     return (int)e;
 }
 
+// nullptr = automatic dispatch; rc = FP8GEMM_OK when the options are usable
+Config config_from_options(const fp8gemm_options* opt, int* rc)
+{
+    *rc = FP8GEMM_OK;
+    if (!opt)
+        return Config{FP8GEMM_KERNEL_AUTO, -1, 0, -1};
+    if (opt->kernel < FP8GEMM_KERNEL_AUTO || opt->kernel > FP8GEMM_KERNEL_SKINNY ||
+        opt->tile_variant >= TILE_VARIANT_COUNT || opt->ksplit < 0 || opt->ksplit > MAX_KSPLIT ||
+        opt->persistent < -1 || opt->persistent > 1)
+        *rc = FP8GEMM_E_KERNEL;
+    return Config{opt->kernel, opt->tile_variant < 0 ? -1 : opt->tile_variant, opt->ksplit, opt->persistent};
+}
+
+// aligned = the plan for 16-byte aligned operands; otherwise the larger of that and what the padded
+// plan needs when every operand has to be copied
+size_t workspace_bytes_for(int m, int n, int k, const Config& cfg, bool any_alignment)
+{
+    if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
+        return 0;
+    const uintptr_t al = 4096;
+    GemmArgs g{reinterpret_cast<const uint8_t*>(al), reinterpret_cast<const uint8_t*>(al),
+               reinterpret_cast<const float*>(al), nullptr, reinterpret_cast<uint16_t*>(al), m, n, k};
+    const Plan p = make_plan(g, cfg);
+    GemmArgs gp = g;
+    gp.m = (m + 15) & ~15;
+    gp.n = (n + 15) & ~15;
+    size_t need = 0;
+    if (p.family >= 0)
+        need = p.padded ? pad_layout(g, plan_workspace_bytes(gp, p), true, false).total : plan_workspace_bytes(g, p);
+    if (any_alignment && !(p.family >= 0 && p.padded)) {
+        // the same shape with an operand off a 16-byte boundary: the plan of the padded shape on copies
+        const long long lim = 0x7FFFFFFFll;
+        if ((long long)gp.m * k <= lim && (long long)gp.n * k <= lim && (long long)gp.m * gp.n <= lim &&
+            cfg.selected != FP8GEMM_KERNEL_SCALAR) {
+            const Plan pp = make_plan(gp, cfg);
+            if (pp.family >= 0 && pp.family != FP8GEMM_KERNEL_SCALAR) {
+                const size_t all = pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total;
+                need = all > need ? all : need;
+            }
+        }
+    }
+    return need;
+}
+
 }  // namespace
 
 extern "C" {
@@ -476,21 +556,38 @@ extern "C" {
 int fp8_block_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
                    int m, int n, int k)
 {
-    return run(a, b, a_scale, b_scale, c, m, n, k, nullptr, g_selected.load());
+    return run(a, b, a_scale, b_scale, c, m, n, k, nullptr, global_config(), nullptr);
 }
 
 int fp8_block_gemm_stream(const void* a, const void* b, const float* a_scale, const float* b_scale,
                           void* c, int m, int n, int k, void* stream)
 {
-    return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream),
-               g_selected.load());
+    return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), global_config(), nullptr);
+}
+
+int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
+                      int m, int n, int k, const fp8gemm_options* options, void* workspace,
+                      size_t workspace_bytes, void* stream)
+{
+    int rc;
+    const Config cfg = config_from_options(options, &rc);
+    if (rc != FP8GEMM_OK)
+        return rc;
+    const Workspace w{static_cast<float*>(workspace), workspace ? workspace_bytes : 0};
+    return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), cfg, &w);
+}
+
+int fp8_block_gemm_ws(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
+                      int m, int n, int k, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return fp8_block_gemm_ex(a, b, a_scale, b_scale, c, m, n, k, nullptr, workspace, workspace_bytes, stream);
 }
 
 int fp8_block_gemm_scalar(const void* a, const void* b, const float* a_scale, const float* b_scale,
                           void* c, int m, int n, int k, void* stream)
 {
     return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream),
-               FP8GEMM_KERNEL_SCALAR);
+               Config{FP8GEMM_KERNEL_SCALAR, -1, 0, -1}, nullptr);
 }
 
 int fp8_block_gemm_select(int kernel_id)
@@ -503,7 +600,7 @@ int fp8_block_gemm_select(int kernel_id)
 
 int fp8_block_gemm_force_config(int tile_variant, int ksplit)
 {
-    if (tile_variant >= TILE_VARIANT_COUNT || ksplit < 0 || ksplit > 64)
+    if (tile_variant >= TILE_VARIANT_COUNT || ksplit < 0 || ksplit > MAX_KSPLIT)
         return FP8GEMM_E_KERNEL;
     g_force_variant.store(tile_variant < 0 ? -1 : tile_variant);
     g_force_ksplit.store(ksplit);
@@ -569,7 +666,7 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
     for (int g = 0; g < groups; ++g) {
         if (m[g] == 0)
             continue;
-        const int rc = run(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k, s, g_selected.load());
+        const int rc = run(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k, s, global_config(), nullptr);
         if (rc != FP8GEMM_OK)
             return rc;
     }
@@ -594,8 +691,9 @@ int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap)
         return FP8GEMM_E_SHAPE;
     // aligned dummy addresses: only their alignment is inspected
     GemmArgs g{reinterpret_cast<const uint8_t*>(uintptr_t(4096)), reinterpret_cast<const uint8_t*>(uintptr_t(4096)),
-               nullptr, nullptr, reinterpret_cast<uint16_t*>(uintptr_t(4096)), m, n, k};
-    Plan p = make_plan(g, g_selected.load());
+               reinterpret_cast<const float*>(uintptr_t(4096)), nullptr, reinterpret_cast<uint16_t*>(uintptr_t(4096)),
+               m, n, k};
+    Plan p = make_plan(g, global_config());
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
     plan_name(p, name, cap);
@@ -604,21 +702,37 @@ int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap)
 
 size_t fp8_block_gemm_workspace_bytes(int m, int n, int k)
 {
-    if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
+    return workspace_bytes_for(m, n, k, global_config(), false);
+}
+
+size_t fp8_block_gemm_workspace_bytes_ex(int m, int n, int k, const fp8gemm_options* options, int any_alignment)
+{
+    int rc;
+    const Config cfg = config_from_options(options, &rc);
+    if (rc != FP8GEMM_OK)
         return 0;
-    // what the plan for 16-byte aligned operands needs under the current selection and forced
-    // configuration; operands with less alignment run kernels that need the same or nothing
-    GemmArgs g{reinterpret_cast<const uint8_t*>(uintptr_t(4096)), reinterpret_cast<const uint8_t*>(uintptr_t(4096)),
-               nullptr, nullptr, reinterpret_cast<uint16_t*>(uintptr_t(4096)), m, n, k};
-    const Plan p = make_plan(g, g_selected.load());
-    if (p.family < 0)
+    return workspace_bytes_for(m, n, k, cfg, any_alignment != 0);
+}
+
+size_t fp8_block_gemm_grouped_workspace_bytes(int groups, const int* m, int n, int k)
+{
+    if (groups <= 0 || !m || n <= 0 || k <= 0 || (k % 128) != 0)
         return 0;
-    if (!p.padded)
-        return plan_workspace_bytes(g, p);
-    GemmArgs gp = g;
-    gp.m = (m + 15) & ~15;
-    gp.n = (n + 15) & ~15;
-    return pad_layout(g, plan_workspace_bytes(gp, p), true, false).total;
+    // the grouped launch on padded copies takes every group's copies at once; one by one the largest
+    // single need would do, which the sum covers
+    const int n16 = (n + 15) & ~15;
+    const size_t nkb = (size_t)k / 128;
+    size_t total = 0;
+    for (int g = 0; g < groups; ++g) {
+        if (m[g] <= 0)
+            continue;
+        const size_t m16 = ((size_t)m[g] + 15) & ~(size_t)15;
+        total += round256((size_t)k * m16) + round256(nkb * m16 * sizeof(float)) + round256((size_t)k * n16) +
+                 round256(m16 * n16 * 2);
+        const size_t single = workspace_bytes_for(m[g], n, k, global_config(), true);
+        total = total > single ? total : single;
+    }
+    return total;
 }
 
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)
@@ -634,16 +748,24 @@ int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)
 int fp8_block_gemm_release(void)
 {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (!g_ws_own && g_ws_retired.empty())
+        return FP8GEMM_OK;
+    hipError_t e = hipDeviceSynchronize();  // kernels of earlier calls may still use the buffers
+    if (e != hipSuccess)
+        return (int)e;
+    hipError_t first = hipSuccess;
+    for (void* p : g_ws_retired) {
+        e = hipFree(p);
+        first = first == hipSuccess ? e : first;
+    }
+    g_ws_retired.clear();
     if (g_ws_own) {
-        hipError_t e = hipDeviceSynchronize();
-        if (e != hipSuccess)
-            return (int)e;
         e = hipFree(g_ws_own);
+        first = first == hipSuccess ? e : first;
         g_ws_own = nullptr;
         g_ws_own_bytes = 0;
-        return (int)e;
     }
-    return FP8GEMM_OK;
+    return (int)first;
 }
 
 int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* stream)
@@ -652,6 +774,8 @@ int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* st
         return FP8GEMM_OK;
     if (!in || !out)
         return FP8GEMM_E_NULLPTR;
+    if (reinterpret_cast<uintptr_t>(in) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 4 != 0)
+        return FP8GEMM_E_ALIGN;  // the kernel reads four floats and writes four codes at a time
     return (int)launch_convert(in, static_cast<uint8_t*>(out), count, static_cast<hipStream_t>(stream));
 }
 
@@ -694,10 +818,10 @@ const char* fp8_block_gemm_error_string(int code)
     case FP8GEMM_E_NULLPTR: return "a required pointer is NULL";
     case FP8GEMM_E_SHAPE: return "m, n, k must be positive and k a multiple of 128";
     case FP8GEMM_E_KERNEL: return "unknown kernel id or kernel not applicable to this shape";
-    case FP8GEMM_E_WORKSPACE: return "workspace too small or misaligned";
+    case FP8GEMM_E_WORKSPACE: return "workspace missing, too small or misaligned (or it would have to grow under stream capture)";
     case FP8GEMM_E_TOOLARGE: return "operand exceeds 2^31-1 elements";
     case FP8GEMM_E_DTYPE: return "unknown source element type";
-    case FP8GEMM_E_ALIGN: return "source pointer is not 16-byte aligned";
+    case FP8GEMM_E_ALIGN: return "pointer alignment: 16 bytes for a source, 4 for the converter's output";
     default: break;
     }
     if (code > 0)
@@ -705,6 +829,6 @@ const char* fp8_block_gemm_error_string(int code)
     return "unknown error code";
 }
 
-int fp8_block_gemm_abi_version(void) { return 2; }
+int fp8_block_gemm_abi_version(void) { return 3; }
 
 }  // extern "C"

@@ -57,18 +57,20 @@ extern "C" int fp8_gemm_host(unsigned short* c, const float* a, const float* b, 
         return rc;
     const float* das = static_cast<const float*>(d_as.p);
     const float* dbs = static_cast<const float*>(d_bs.p);
-    if (option == 2) {
-        rc = fp8_block_gemm_scalar(d_a8.p, d_b8.p, das, dbs, d_c.p, (int)m, (int)n, (int)k, nullptr);
-    } else if (option == 0 || option == 1) {
-        rc = fp8_block_gemm(d_a8.p, d_b8.p, das, dbs, d_c.p, (int)m, (int)n, (int)k);
-    } else if (option >= 100 && option <= 100 + FP8GEMM_KERNEL_SKINNY) {
-        rc = fp8_block_gemm_select(option - 100);
-        if (rc == 0)
-            rc = fp8_block_gemm(d_a8.p, d_b8.p, das, dbs, d_c.p, (int)m, (int)n, (int)k);
-        (void)fp8_block_gemm_select(FP8GEMM_KERNEL_AUTO);
-    } else {
+    // per-call options and a workspace of this call's own: no process-wide switch is touched
+    fp8gemm_options opt{FP8GEMM_KERNEL_AUTO, -1, 0, -1};
+    if (option == 2)
+        opt.kernel = FP8GEMM_KERNEL_SCALAR;
+    else if (option >= 100 && option <= 100 + FP8GEMM_KERNEL_SKINNY)
+        opt.kernel = option - 100;
+    else if (option != 0 && option != 1)
         return FP8GEMM_E_KERNEL;
-    }
+    const size_t ws_bytes = fp8_block_gemm_workspace_bytes_ex((int)m, (int)n, (int)k, &opt, 0);
+    DeviceBuf d_ws;
+    if (ws_bytes)
+        TRY(d_ws.alloc(ws_bytes));
+    rc = fp8_block_gemm_ex(d_a8.p, d_b8.p, das, dbs, d_c.p, (int)m, (int)n, (int)k, &opt, d_ws.p, ws_bytes,
+                           nullptr);
     if (rc != 0)
         return rc;
     TRY(hipMemcpy(c, d_c.p, m * n * 2, hipMemcpyDeviceToHost));  // blocking: also the sync

@@ -16,8 +16,10 @@ __global__ void __launch_bounds__(256) scalar_gemm_kernel(const uint8_t* __restr
     // no fused multiply-add anywhere but the explicit fmaf below: "result += block * as * bs"
     // keeps its three separately rounded operations, as in a CPU build of the same line
 #pragma clang fp contract(off)
-    int col = blockIdx.x * 64 + (threadIdx.x & 63);
-    int row = blockIdx.y * 4 + (threadIdx.x >> 6);
+    // rows ride on grid.x, whose limit (2^31 - 1 blocks) no accepted m reaches; grid.y carries the
+    // 64-column strips, of which the validation's 2^31 - 1 element bound on m*n leaves few when m is large
+    int col = blockIdx.y * 64 + (threadIdx.x & 63);
+    int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= m || col >= n)
         return;
     int sn = (n + KBLOCK - 1) / KBLOCK;
@@ -38,7 +40,10 @@ __global__ void __launch_bounds__(256) scalar_gemm_kernel(const uint8_t* __restr
 
 hipError_t launch_scalar(const GemmArgs& g, hipStream_t s)
 {
-    dim3 grid((g.n + 63) / 64, (g.m + 3) / 4);
+    const unsigned strips = (unsigned)((g.n + 63) / 64);
+    if (strips > 65535u)  // n beyond 4 M columns: not a shape this kernel is for
+        return hipErrorInvalidConfiguration;
+    dim3 grid((unsigned)((g.m + 3) / 4), strips);
     hipLaunchKernelGGL(scalar_gemm_kernel, grid, dim3(256), 0, s, g.a, g.b, g.a_scale, g.b_scale,
                        g.c, g.m, g.n, g.k);
     return hipGetLastError();

@@ -208,10 +208,7 @@ hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s)
     hipError_t e;
     if (ksplit > 1) {
         auto kern = skinny_gemm_kernel<true>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS);
-        if (e != hipSuccess)
-            return e;
+        FP8GEMM_ALLOW_LDS(kern, SK_LDS);
         hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), SK_LDS, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, g.n, g.k, tiles_n, kb_per_split);
         e = hipGetLastError();
@@ -220,10 +217,7 @@ hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s)
         return launch_splitk_reduce(g, ksplit, partial, s);
     }
     auto kern = skinny_gemm_kernel<false>;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS);
-    if (e != hipSuccess)
-        return e;
+    FP8GEMM_ALLOW_LDS(kern, SK_LDS);
     hipLaunchKernelGGL(kern, grid, dim3(SK_THREADS), SK_LDS, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
                        partial, g.m, g.n, g.k, tiles_n, kb_per_split);
     return hipGetLastError();

@@ -430,21 +430,14 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStre
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     dim3 grid(tiles_m * tiles_n, ksplit);
     const int group_m = choose_group_m(tiles_m, tiles_n, BM, BN);
-    hipError_t e;
     if (ksplit > 1) {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
-        if (e != hipSuccess)
-            return e;
+        FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
     } else {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
-        if (e != hipSuccess)
-            return e;
+        FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
                            g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
     }

@@ -602,10 +602,7 @@ hipError_t launch_persistent_variant(const GemmArgs& g, int workgroups, hipStrea
     constexpr int LDS_TOTAL = S::LDS_BYTES + (WM * WN == 4 ? PR * (BN * 2 + 8) : 0);
     const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     auto kern = tile_gemm_persistent_kernel<BM, BN, WM, WN, NS, PR>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
-    if (e != hipSuccess)
-        return e;
+    FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
     hipLaunchKernelGGL(kern, dim3(workgroups), dim3(64 * WM * WN), LDS_TOTAL, s, g.a, g.b, g.a_scale,
                        g.b_scale, g.c, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n);
     return hipGetLastError();
@@ -621,10 +618,7 @@ hipError_t launch_grouped_variant(GroupTable& tab, int n, int k, int workgroups,
     for (int g = 0; g < tab.groups; ++g)
         tab.tile_start[g + 1] = tab.tile_start[g] + ((tab.m[g] + BM - 1) / BM) * tiles_n;
     auto kern = tile_gemm_grouped_kernel<BM, BN, WM, WN, NS, PR>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_TOTAL);
-    if (e != hipSuccess)
-        return e;
+    FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
     hipLaunchKernelGGL(kern, dim3(workgroups), dim3(NTHREADS), LDS_TOTAL, s, tab, n, k, tiles_n);
     return hipGetLastError();
 }

@@ -5,6 +5,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fp8gemm {
 
 struct GemmArgs {
@@ -19,6 +21,26 @@ struct GemmArgs {
     int lda = 0;
 };
 inline int leading_dim(const GemmArgs& g) { return g.lda ? g.lda : g.m; }
+
+// Kernels with more than 64 KiB of dynamic LDS need the attribute raised before their first launch
+// on a device.  Once per kernel and device (a bit per device in a word the call site owns) instead of
+// once per launch: the runtime call costs as much as a short kernel takes.
+#define FP8GEMM_ALLOW_LDS(kern, bytes)                                                                       \
+    do {                                                                                                     \
+        static std::atomic<uint64_t> done_{0};                                                               \
+        int dev_ = 0;                                                                                        \
+        hipError_t e_ = hipGetDevice(&dev_);                                                                 \
+        if (e_ != hipSuccess)                                                                                \
+            return e_;                                                                                       \
+        const uint64_t bit_ = 1ull << (dev_ & 63);                                                           \
+        if (!(done_.load(std::memory_order_acquire) & bit_)) {                                               \
+            e_ = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                    \
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (bytes));                   \
+            if (e_ != hipSuccess)                                                                            \
+                return e_;                                                                                   \
+            done_.fetch_or(bit_, std::memory_order_release);                                                 \
+        }                                                                                                    \
+    } while (0)
 
 // one thread per C element (check.cu:30-49)
 hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);

@@ -16,8 +16,15 @@
  *
  * Return value: 0 on success; a negative FP8GEMM_E_* code for argument errors, detected
  * before any device call; a positive hipError_t value when the HIP runtime reports one.
- * Nothing is thrown across this boundary.  Launches are asynchronous on the given stream;
- * no entry point synchronises the device.
+ * Nothing is thrown across this boundary.  Launches are asynchronous on the given stream; no
+ * entry point waits for the device except fp8_block_gemm_release and fp8_gemm_host.
+ *
+ * Threads and streams.  fp8_block_gemm_ex / fp8_block_gemm_ws take everything they depend on as
+ * arguments (options, workspace, stream) and read no process-wide state: any number of host
+ * threads may call them at once, on any streams, as long as calls that run concurrently on the
+ * device use different workspaces.  The shorter entry points use process-wide defaults
+ * (fp8_block_gemm_select, _force_config, _set_persistent: meant for tests, benchmarks and drivers
+ * that mirror the reference's compile-time switches) and ONE process-wide workspace.
  */
 #ifndef FP8_BLOCK_GEMM_H
 #define FP8_BLOCK_GEMM_H
@@ -32,10 +39,11 @@ extern "C" {
 #define FP8GEMM_E_NULLPTR (-1)   /* a required pointer is NULL */
 #define FP8GEMM_E_SHAPE (-2)     /* m, n or k <= 0, or k not a multiple of 128 */
 #define FP8GEMM_E_KERNEL (-3)    /* unknown kernel id, or the kernel cannot run this shape */
-#define FP8GEMM_E_WORKSPACE (-4) /* caller-provided workspace too small or misaligned */
+#define FP8GEMM_E_WORKSPACE (-4) /* workspace missing, too small or misaligned; or the library-owned one
+                                    would have to be (re)allocated while the stream is being captured */
 #define FP8GEMM_E_TOOLARGE (-5)  /* m*k, n*k or m*n does not fit the 32-bit offsets used */
 #define FP8GEMM_E_DTYPE (-6)     /* unknown FP8GEMM_DTYPE_* value */
-#define FP8GEMM_E_ALIGN (-7)     /* a source pointer is not 16-byte aligned */
+#define FP8GEMM_E_ALIGN (-7)     /* a source pointer is not 16-byte aligned (converter: output not 4-byte aligned) */
 
 /* Element type of a quantiser's source matrix, and with it the arithmetic: quantize.py computes
  * in the tensor's own dtype, i.e. torch rounds every element-wise result to bf16 for a bf16
@@ -83,8 +91,9 @@ int fp8_block_gemm_scalar(const void* a, const void* b, const float* a_scale,
 int fp8_block_gemm_select(int kernel_id);
 
 /* Pin the MFMA tile kernels to one workgroup tile (0 = 256x192, 1 = 256x128, 2 = 128x128,
- * 3 = 128x192, 4 = 64x64 rows x columns of C; -1 = choose by cost model) and one K-split
- * count (0 = choose).  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
+ * 3 = 128x192, 4 = 64x64 rows x columns of C, 5 = 256x192 with one wave per SIMD (persistent
+ * form only, never chosen automatically); -1 = choose by cost model) and one K-split count
+ * (0 = choose, at most 16; more returns FP8GEMM_E_KERNEL).  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
  * (/root/reference/mn_large.hip:1-8). */
 int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 
@@ -110,34 +119,67 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
                            const float* const* a_scale, const float* const* b_scale,
                            void* const* c, const int* m, int n, int k, void* stream);
 
+/* Per-call form.  `options` (NULL = automatic dispatch) replaces the process-wide switches above for
+ * this call only; `workspace` (256-byte aligned device memory of `workspace_bytes`; NULL / 0 when the
+ * plan needs none) replaces the process-wide workspace: the call allocates nothing, synchronises
+ * nothing and returns FP8GEMM_E_WORKSPACE when the plan needs more than it was given
+ * (fp8_block_gemm_workspace_bytes_ex tells how much).  Safe to call from several host threads and on
+ * several streams at once with distinct workspaces, and under stream capture.  No counterpart in the
+ * reference, whose launcher is single-threaded on stream 0 (/root/reference/check.cu:106-119). */
+typedef struct fp8gemm_options {
+    int kernel;       /* FP8GEMM_KERNEL_* */
+    int tile_variant; /* as fp8_block_gemm_force_config; -1 = cost model */
+    int ksplit;       /* 0 = cost model, else 1..16 */
+    int persistent;   /* as fp8_block_gemm_set_persistent */
+} fp8gemm_options;
+int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
+                      int m, int n, int k, const fp8gemm_options* options, void* workspace,
+                      size_t workspace_bytes, void* stream);
+/* fp8_block_gemm_ex with automatic dispatch. */
+int fp8_block_gemm_ws(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
+                      int m, int n, int k, void* workspace, size_t workspace_bytes, void* stream);
+/* Workspace bytes fp8_block_gemm_ex needs for (m, n, k) under `options` (NULL = automatic).
+ * any_alignment = 0: for a, b, a_scale, c on 16-byte boundaries (what allocators return);
+ * any_alignment != 0: an upper bound that also covers operands off such a boundary, which run on
+ * padded copies of every operand concerned (for cfg-sized shapes that is the size of all operands).
+ * Touches no device.  0 for an invalid shape or options. */
+size_t fp8_block_gemm_workspace_bytes_ex(int m, int n, int k, const fp8gemm_options* options,
+                                         int any_alignment);
+
 /* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
  * 16-byte aligned operands into name[0..cap), e.g. "tile256x192_k1_persistent", "tile128x128_k3", "skinny_k1", "padded_tile64x64_k1", "scalar".
  * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart
  * in the reference (its choice is made by editing the source, README.md:55). */
 int fp8_block_gemm_plan(int m, int n, int k, char* name, size_t cap);
 
-/* Name of the kernel variant the last successful call on this thread launched
+/* Name of the kernel plan the last successful GEMM call on this thread launched
  * (static storage, never NULL).  No counterpart in the reference: diagnostics. */
 const char* fp8_block_gemm_last_kernel(void);
 
-/* Split-K kernels keep fp32 partial tiles in device memory.  By default the library owns a
- * lazily grown buffer (allocated on first need, kept until fp8_block_gemm_release).
- * A caller that must not allocate can supply its own, 256-byte aligned, of at least
- * fp8_block_gemm_workspace_bytes(m, n, k) bytes for every shape it will pass: that is what
- * the plan for the shape needs under the kernel selection and forced configuration in force
- * when it is asked (0 when the plan neither splits K nor pads; for a padded plan an upper bound that holds for
- * any operand alignment; ask again after changing either).
- * Passing NULL returns to the library-owned buffer.  There is ONE workspace per process,
- * on the device that was current when it was allocated or supplied: calls that split K
- * (fp8_block_gemm_plan names them "..._kN" with N > 1) or run on padded copies ("padded_...")
- * must not overlap on different streams, and must run on that device; other calls never
- * touch it.  The reference has
- * no workspace (its kernels do not split K: mn_small.hip:28). */
+/* The process-wide workspace of the entry points without a workspace argument.  Plans that split K
+ * ("..._kN", N > 1) keep fp32 partial tiles there, plans for operands off the 16-byte grid
+ * ("padded_...") their copies; other plans never touch it.  By default the library owns a buffer that
+ * it allocates on first need and replaces by a larger one when a call needs more; the outgrown buffer
+ * is kept until fp8_block_gemm_release, so kernels in flight and graphs captured earlier stay valid --
+ * but a graph replays into the buffer it was captured with, which later calls no longer share: give
+ * captured work a workspace of its own.  A call that would have to allocate while its stream is being
+ * captured returns FP8GEMM_E_WORKSPACE and leaves the capture valid.
+ * fp8_block_gemm_set_workspace supplies a caller-owned buffer instead (256-byte aligned; NULL returns
+ * to the library-owned one); it must hold fp8_block_gemm_workspace_bytes(m, n, k) for every shape
+ * passed: what the plan needs under the switches in force when asked, for 16-byte aligned operands
+ * (0 when the plan neither splits K nor pads; operands off a 16-byte boundary need what
+ * fp8_block_gemm_workspace_bytes_ex(m, n, k, NULL, 1) returns).  fp8_block_gemm_grouped_workspace_bytes
+ * bounds what fp8_block_gemm_grouped takes for any alignment; with a smaller caller-owned buffer the
+ * groups run one by one.  There is ONE such workspace per process, on the device that was current when
+ * it was allocated or supplied: calls that use it must not overlap on different streams.  The reference
+ * has no workspace (its kernels do not split K: mn_small.hip:28). */
 size_t fp8_block_gemm_workspace_bytes(int m, int n, int k);
+size_t fp8_block_gemm_grouped_workspace_bytes(int groups, const int* m, int n, int k);
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes);
 int fp8_block_gemm_release(void);
 
-/* fp32 -> fp8 e4m3fn, round to nearest even, saturating to +-448; count elements.
+/* fp32 -> fp8 e4m3fn, round to nearest even, saturating to +-448; count elements; `in` 16-byte and
+ * `out` 4-byte aligned (FP8GEMM_E_ALIGN otherwise).
  * Replaces convert_float_to_fp8<<<M*K/256, 256>>> (/root/reference/check.cu:17-22, 83-84);
  * unlike that launch it also converts a tail that is not a multiple of 256. */
 int fp8_convert_f32_to_e4m3fn(const float* in, void* out, size_t count, void* stream);

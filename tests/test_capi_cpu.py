@@ -10,10 +10,11 @@ import pytest
 def test_library_exports_every_declared_symbol(pkg):
     L = pkg.lib()
     names = pkg.abi_symbols()
-    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and len(names) == 18
+    assert "fp8_block_gemm" in names and "fp8_gemm_host" in names and "fp8_block_gemm_ex" in names
+    assert len(names) >= 22
     for name in names:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
-    assert L.fp8_block_gemm_abi_version() == 2
+    assert L.fp8_block_gemm_abi_version() == 3
 
 
 def test_argument_validation_happens_before_any_device_call(pkg):
@@ -31,6 +32,8 @@ def test_argument_validation_happens_before_any_device_call(pkg):
     assert L.fp8_gemm_host(p, p, p, p, p, 16, 16, 130, 0) == -2
     assert L.fp8_convert_f32_to_e4m3fn(None, p, 10, None) == -1
     assert L.fp8_convert_f32_to_e4m3fn(None, None, 0, None) == 0
+    assert L.fp8_convert_f32_to_e4m3fn(p + 4, p, 10, None) == -7     # float4 loads need 16-byte alignment
+    assert L.fp8_convert_f32_to_e4m3fn(p, p + 2, 10, None) == -7     # 4-byte stores
     for fn in (L.fp8_quantize_a_1x128, L.fp8_quantize_b_128x128):
         assert fn(None, 0, p, p, 16, 128, None) == -1
         assert fn(p, 0, p, None, 16, 128, None) == -1
@@ -73,6 +76,8 @@ def test_select_and_force_config_validate(pkg):
     assert L.fp8_block_gemm_select(-1) == -3
     assert L.fp8_block_gemm_force_config(99, 0) == -3
     assert L.fp8_block_gemm_force_config(0, 1000) == -3
+    assert L.fp8_block_gemm_force_config(0, 17) == -3                # the dispatcher splits K at most 16 times
+    assert L.fp8_block_gemm_force_config(0, 16) == 0
     for kid in (1, 2, 3, 4, 0):
         assert L.fp8_block_gemm_select(kid) == 0
     assert L.fp8_block_gemm_force_config(-1, 0) == 0
@@ -103,6 +108,64 @@ def test_workspace_contract(pkg):
     assert L.fp8_block_gemm_set_workspace(4096 + 8, 1 << 20) == -4   # misaligned
     assert L.fp8_block_gemm_set_workspace(None, 0) == 0
     assert L.fp8_block_gemm_release() == 0                           # nothing allocated yet
+
+
+def test_per_call_entry_point_validates_and_never_allocates(pkg):
+    """fp8_block_gemm_ex / _ws: bad options and a missing workspace are host-side errors, reported
+    before any device call (the pointers below are never dereferenced)."""
+    L = pkg.lib()
+    p = 4096
+    O = pkg.Options
+    assert L.fp8_block_gemm_ex(p, p, p, p, p, 16, 16, 100, None, None, 0, None) == -2
+    assert L.fp8_block_gemm_ex(None, p, p, p, p, 16, 16, 128, None, None, 0, None) == -1
+    for bad in (O(kernel=9), O(tile_variant=99), O(ksplit=17), O(ksplit=-1), O(persistent=2)):
+        assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(bad), None, 0, None) == -3
+        assert pkg.workspace_bytes_ex(256, 256, 1024, bad) == 0
+    split = O(kernel=pkg.KERNEL_SPLITK, tile_variant=2, ksplit=4)
+    need = pkg.workspace_bytes_ex(256, 256, 1024, split)
+    assert need == 4 * 256 * 256 * 4
+    # a plan that needs a workspace and is not given one (or too little, or a misaligned one)
+    assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(split), None, 0, None) == -4
+    assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(split), p, need - 1, None) == -4
+    assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(split), p + 16, need, None) == -4
+    # operands off a 16-byte boundary run on padded copies: the aligned figure is not enough, and says so
+    assert L.fp8_block_gemm_ws(p + 1, p, p, p, p, 256, 256, 1024, p, 1024, None) == -4
+    # the per-call options do not leak into, or read, the process-wide switches
+    pkg.force_config(1, 4)
+    try:
+        assert pkg.workspace_bytes_ex(1024, 512, 2048) == pkg.workspace_bytes_ex(1024, 512, 2048, O())
+        assert pkg.workspace_bytes(1024, 512, 2048) == 4 * 1024 * 512 * 4
+    finally:
+        pkg.force_config(-1, 0)
+
+
+def test_workspace_queries_cover_every_alignment(pkg):
+    for (m, n, k) in [(256, 256, 1024), (1024, 512, 7168), (8192, 4608, 7168), (33, 100, 128), (32, 7168, 2048)]:
+        aligned = pkg.workspace_bytes_ex(m, n, k)
+        anyal = pkg.workspace_bytes_ex(m, n, k, None, True)
+        assert anyal >= aligned
+        m16, n16 = (m + 15) // 16 * 16, (n + 15) // 16 * 16
+        copies = k * m16 + (k // 128) * m16 * 4 + k * n16 + m16 * n16 * 2
+        assert anyal >= copies, (m, n, k)
+    # grouped: at least the copies of every group, and at least any single group's need
+    ms = [509, 1027, 771]
+    tot = pkg.grouped_workspace_bytes(ms, 7168, 2048)
+    assert tot >= sum(2048 * ((x + 15) // 16 * 16) for x in ms)
+    assert tot >= max(pkg.workspace_bytes_ex(x, 7168, 2048, None, True) for x in ms)
+    assert pkg.grouped_workspace_bytes([], 7168, 2048) == 0
+
+
+def test_one_wave_per_simd_variant_is_opt_in(pkg):
+    assert "w4" not in pkg.plan(8192, 4608, 7168)
+    pkg.force_config(5, 0)
+    try:
+        assert pkg.plan(8192, 4608, 7168) == "tile256x192w4_k1_persistent"
+        assert pkg.plan(256, 192, 128) == "tile256x192w4_k1_persistent"   # exists in the persistent form only
+        pkg.force_config(5, 2)
+        with pytest.raises(pkg.Fp8GemmError):
+            pkg.plan(1024, 512, 2048)                                     # and without a K split
+    finally:
+        pkg.force_config(-1, 0)
 
 
 def test_dispatcher_plans(pkg):

@@ -57,6 +57,30 @@ def _assert_close(got, ref, what):
     return r
 
 
+def _assert_every_element(got, a, b, sa, sb, m, n, k, what):
+    """A bound per element, tight enough to see one lost or doubled K block anywhere:
+
+        |C - ref| <= 2^-7 |ref| + 2^-12 S,   S = sum over K blocks of scale * sum |a| |b|
+
+    ref = the oracle's fp32 value before its bf16 cast.  2^-7 |ref| = one bf16 ulp (the output
+    rounding, and a neighbouring code when the two fp32 sums straddle a rounding boundary);
+    2^-12 S bounds what a different summation order inside the blocks can move, also where the
+    terms cancel (the oracle's sequential fp32 sum and the matrix unit's accumulation each stay
+    within about 2^-16 S of the exact sum; with 1 % of the entries fifty times larger the measured
+    worst case is 2^-13.7 S).  One missing K block of 56 moves a typical element by 2.5e-3 S
+    against a bound of about 4e-4 S."""
+    _, ref32 = oracle.ref_gemm(a, b, sa, sb, m, n, k, want_f32=True)
+    _, s32 = oracle.ref_gemm(a & 0x7F, b & 0x7F, np.abs(sa), np.abs(sb), m, n, k, want_f32=True)
+    c = oracle.bf16_decode(got).astype(np.float64).reshape(m, n)
+    err = np.abs(c - ref32.astype(np.float64))
+    bound = 2.0 ** -7 * np.abs(ref32.astype(np.float64)) + 2.0 ** -12 * s32.astype(np.float64)
+    ratio = err / np.maximum(bound, 1e-30)
+    worst = np.unravel_index(np.argmax(ratio), ratio.shape)
+    _say(f"[gpu case] {what}: per-element bound, worst err/bound = {ratio[worst]:.3f} at {worst}")
+    assert np.isfinite(c).all(), what
+    assert (err <= bound).all(), (what, worst, float(err[worst]), float(bound[worst]))
+
+
 # ------------------------------------------------------------------ scalar definition kernel
 @pytest.mark.parametrize("m,n,k", [(1, 1, 128), (48, 80, 128), (64, 128, 256), (33, 130, 384),
                                    (128, 128, 256)])
@@ -90,6 +114,7 @@ def test_tile_kernel(pkg, variant, m, n, k):
     got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant)
     assert name.endswith("_k1"), name
     _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
 
 
 # persistent form: several tiles per workgroup (more than 256 tiles), ragged edges, K ranges from
@@ -124,6 +149,7 @@ def test_tile_kernel_one_wave_per_simd(pkg, m, n, k):
     got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=5)
     assert name == "tile256x192w4_k1_persistent", name
     _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
     plain, name0 = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=0, persistent=0)
     assert name0 == "tile256x192_k1", name0
     assert np.array_equal(got, plain), "both forms fold the same block sums in the same order"
@@ -211,6 +237,24 @@ def test_benchmark_config_full_size(pkg, name):
     r = _assert_close(got, ref, f"{name} {kname}")
     _say(f"[gpu case] {name} {kname}: max_err={r['max_err']:.4g} bound={r['bound']:.4g}")
     assert kname != "scalar"
+    _assert_every_element(got, a, b, sa, sb, m, n, k, f"{name} {kname}")
+
+
+# the 18 shapes of the reference's results table (/root/reference/README.md:15-25), which the
+# dispatcher's cost model and table were fitted on: automatic dispatch against the whole oracle result
+CHALLENGE_KN = [(7168, 1536), (1536, 3072), (7168, 576), (256, 7168), (2048, 7168), (7168, 4608),
+                (2304, 7168), (7168, 512), (512, 4096)]
+
+
+@pytest.mark.parametrize("m", [1024, 6144])
+@pytest.mark.parametrize("k,n", CHALLENGE_KN)
+def test_challenge_shapes_under_automatic_dispatch(pkg, m, k, n):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 9000 + m + n + k)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, kname = _run(pkg, a, b, sa, sb, m, n, k)
+    assert kname == pkg.plan(m, n, k) and kname != "scalar", kname
+    _assert_close(got, ref, f"{m}x{n}x{k} {kname}")
+    _assert_every_element(got, a, b, sa, sb, m, n, k, f"{m}x{n}x{k} {kname}")
 
 
 # ------------------------------------------------------------------ size-independent properties
