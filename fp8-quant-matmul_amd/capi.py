@@ -70,6 +70,8 @@ def lib():
     L.fp8_block_gemm_workspace_bytes_ex.argtypes = [i, i, i, C.POINTER(Options), i]
     L.fp8_block_gemm_grouped_workspace_bytes.restype = sz
     L.fp8_block_gemm_grouped_workspace_bytes.argtypes = [i, C.POINTER(C.c_int), i, i]
+    L.fp8_block_gemm_noalloc.restype = i
+    L.fp8_block_gemm_noalloc.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
     L.fp8_block_gemm_scalar.restype = i
     L.fp8_block_gemm_scalar.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
     L.fp8_block_gemm_select.restype = i
@@ -142,6 +144,16 @@ def gemm_ex(a, b, a_scale, b_scale, c, m, n, k, options=None, workspace=None, wo
     rc = lib().fp8_block_gemm_ex(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k, opt,
                                  _ptr(workspace), workspace_bytes, stream)
     _check(rc, "fp8_block_gemm_ex")
+
+
+NOALLOC_MAX_BYTES = 32 << 20
+
+
+def gemm_noalloc(a, b, a_scale, b_scale, c, m, n, k, stream=None):
+    """fp8_block_gemm_stream with the library's fixed in-image workspace: allocates nothing; plans that
+    need more than NOALLOC_MAX_BYTES raise (code -4)."""
+    _check(lib().fp8_block_gemm_noalloc(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(c), m, n, k,
+                                        stream), "fp8_block_gemm_noalloc")
 
 
 def workspace_bytes_ex(m, n, k, options=None, any_alignment=False):

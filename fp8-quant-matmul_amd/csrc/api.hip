@@ -404,6 +404,36 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
     return rc;
 }
 
+// ---- the entry point that allocates nothing: its workspace is this array, part of the library's device
+// image (every GPU the library runs on holds its own copy, at its own address, until the process
+// ends).  In host code the array's name is only a handle for hipGetSymbolAddress: the device address is
+// looked up once per device, with that device current, and everything else uses that pointer.
+static __device__ __align__(256) unsigned char scratch[FP8GEMM_NOALLOC_MAX_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+int scratch_for_current_device(void** out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES)
+        return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess)
+            return (int)e;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return FP8GEMM_OK;
+}
+
 // tile shape for a grouped launch: what the cost model picks for the stacked problem, among the
 // shapes that have a persistent form, without a K split; -1 when none can take the table
 int grouped_variant(const GroupTable& tab, int n, int k)
@@ -581,6 +611,31 @@ int fp8_block_gemm_ws(const void* a, const void* b, const float* a_scale, const 
                       int m, int n, int k, void* workspace, size_t workspace_bytes, void* stream)
 {
     return fp8_block_gemm_ex(a, b, a_scale, b_scale, c, m, n, k, nullptr, workspace, workspace_bytes, stream);
+}
+
+int fp8_block_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
+                           int m, int n, int k, void* stream)
+{
+    // arguments first (no device call), then the plan's need against the fixed size: a plan that does
+    // not fit is refused here, with the code a too small workspace always gets
+    const int v = validate(a, b, a_scale, b_scale, c, m, n, k);
+    if (v != FP8GEMM_OK)
+        return v;
+    const Config cfg = global_config();
+    const GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), a_scale, b_scale,
+                     static_cast<uint16_t*>(c), m, n, k};
+    const Plan p = make_plan(g, cfg);
+    if (p.family < 0)
+        return FP8GEMM_E_KERNEL;
+    const size_t need = p.padded ? padded_bytes(g, p) : plan_workspace_bytes(g, p);
+    if (need > (size_t)FP8GEMM_NOALLOC_MAX_BYTES)
+        return FP8GEMM_E_WORKSPACE;
+    void* ptr = nullptr;
+    const int rc = scratch_for_current_device(&ptr);
+    if (rc != FP8GEMM_OK)
+        return rc;
+    const Workspace w{static_cast<float*>(ptr), (size_t)FP8GEMM_NOALLOC_MAX_BYTES};
+    return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), cfg, &w);
 }
 
 int fp8_block_gemm_scalar(const void* a, const void* b, const float* a_scale, const float* b_scale,

@@ -146,6 +146,20 @@ int fp8_block_gemm_ws(const void* a, const void* b, const float* a_scale, const 
 size_t fp8_block_gemm_workspace_bytes_ex(int m, int n, int k, const fp8gemm_options* options,
                                          int any_alignment);
 
+/* fp8_block_gemm_stream for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same dispatch under the same process-wide switches, but
+ * the workspace of plans that split K or pad is a fixed array inside the library's device image,
+ * FP8GEMM_NOALLOC_MAX_BYTES per GPU, held until the process ends.  The call allocates and frees nothing.
+ * A plan that needs more than that returns FP8GEMM_E_WORKSPACE (ask fp8_block_gemm_workspace_bytes /
+ * _ex beforehand; plans that neither split K nor pad need nothing and always fit).  All calls on one
+ * GPU share that GPU's array: calls that use it and overlap on the device (different streams) race, as
+ * with the process-wide workspace.  Nothing in it has to start at zero: every plan writes what it later
+ * reads.  The first call on a device looks the array's address up (hipGetSymbolAddress); make that call
+ * outside a stream capture.  This entry point has no counterpart in the reference. */
+#define FP8GEMM_NOALLOC_MAX_BYTES (32u << 20)
+int fp8_block_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                           void* c, int m, int n, int k, void* stream);
+
 /* Writes the name of the kernel plan the dispatcher would launch for (m, n, k) with
  * 16-byte aligned operands into name[0..cap), e.g. "tile256x192_k1_persistent", "tile128x128_k3", "skinny_k1", "padded_tile64x64_k1", "scalar".
  * Touches no device.  Returns 0, or a negative code for an invalid shape.  No counterpart

@@ -155,6 +155,23 @@ def test_workspace_queries_cover_every_alignment(pkg):
     assert pkg.grouped_workspace_bytes([], 7168, 2048) == 0
 
 
+def test_noalloc_entry_point_validates_before_any_device_call(pkg):
+    L = pkg.lib()
+    p = 4096
+    assert L.fp8_block_gemm_noalloc(None, p, p, p, p, 16, 16, 128, None) == -1
+    assert L.fp8_block_gemm_noalloc(p, p, p, p, p, 16, 16, 100, None) == -2
+    assert L.fp8_block_gemm_noalloc(p, p, p, p, p, 70000, 16, 65536, None) == -5
+    # a plan whose partial sums exceed the fixed array: refused by size, no device touched
+    pkg.select(pkg.KERNEL_SPLITK)
+    pkg.force_config(2, 4)
+    try:
+        assert pkg.workspace_bytes(4096, 4096, 1024) > pkg.NOALLOC_MAX_BYTES
+        assert L.fp8_block_gemm_noalloc(p, p, p, p, p, 4096, 4096, 1024, None) == -4
+    finally:
+        pkg.select(0)
+        pkg.force_config(-1, 0)
+
+
 def test_one_wave_per_simd_variant_is_opt_in(pkg):
     assert "w4" not in pkg.plan(8192, 4608, 7168)
     pkg.force_config(5, 0)
