@@ -209,6 +209,30 @@ def main():
         ts.sort()
         return ts[len(ts) // 2]
 
+    def rotating_operand_us(dev, dc, shape, min_bytes=640 << 20, launches=600):
+        """Launches back to back, each on another copy of B: more copies than the part's 256 MB
+        Infinity Cache and its L2s hold together (`min_bytes` of B in total), so B comes from HBM every
+        time, as the weights of successive layers do in a decode step.  No fill kernel, no idle gap."""
+        m_, n_, k_ = shape
+        copies = max(2, -(-min_bytes // (n_ * k_)))
+        bs = [dev[1]] + [dev[1].clone() for _ in range(copies - 1)]
+        call = lambda i: pkg.gemm(dev[0], bs[i % copies], dev[2], dev[3], dc, m_, n_, k_, sptr)
+        for i in range(2 * copies):
+            call(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        for i in range(copies):          # the queue is busy when the first event is reached
+            call(i)
+        e0.record(stream)
+        for i in range(launches):
+            call(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / launches
+        del bs
+        return us, copies
+
     def shape_report(name, steps, warmup, exact=False):
         shape, host, dev, dc = prepare(name)
         step(dev, dc, shape)
@@ -231,6 +255,12 @@ def main():
             cold = cold_latency_us(dev, dc, shape)
             rep["cold_latency_us"] = round(cold, 2)
             rep["cold_gbs"] = round(byts / cold * 1e-3, 1)
+        if name in HBM_BOUND:
+            # the HBM-side figure: B from HBM on every launch (rotating copies), launches back to back
+            rot_us, copies = rotating_operand_us(dev, dc, shape)
+            rep["hbm_rotating"] = {"b_copies": copies, "b_bytes_total": copies * shape[1] * shape[2],
+                                   "latency_us": round(rot_us, 2), "gbs": round(byts / rot_us * 1e-3, 1),
+                                   "frac_hbm_peak": round(byts / rot_us * 1e-3 / PEAK_HBM_GBS, 4)}
         if not args.no_cpu and not isinstance(name, tuple):
             rep["cpu"] = cpu_row(shape, host)
         return rep, (shape, host, wall_ms, ev_ms)
