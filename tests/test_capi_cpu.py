@@ -220,3 +220,16 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True,
                        text=True, timeout=120)
     assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_generated_k_loop_is_what_its_generator_writes():
+    """csrc/w4_loop.inc (the assembly K loop of tile variant 5) is committed generated text: it has to be
+    exactly what csrc/gen_w4_loop.py prints, or the library was built from something nobody can regenerate"""
+    import os
+    import subprocess
+    import sys
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "fp8-quant-matmul_amd", "csrc")
+    out = subprocess.run([sys.executable, os.path.join(csrc, "gen_w4_loop.py")], capture_output=True, text=True,
+                         check=True).stdout
+    with open(os.path.join(csrc, "w4_loop.inc")) as f:
+        assert f.read() == out
