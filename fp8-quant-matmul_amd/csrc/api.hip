@@ -128,7 +128,10 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit)
     const double per_kb = 1.19 * area + 0.267;
     const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     const long items = (long)tiles * ksplit;
-    const long rounds = (items + NUM_CU - 1) / NUM_CU;
+    // two 64x64 workgroups share a CU; counted only for a single row of tiles (M <= 64), where the K
+    // split decides everything: the constants above were fitted to taller problems without it
+    const long slots = (variant == TILE_64x64 && g.m <= 64) ? 2 * NUM_CU : NUM_CU;
+    const long rounds = (items + slots - 1) / slots;
     double cost = 1.79 + rounds * per_item;
     if (ksplit > 1)  // second launch + partial write and read-back
         cost += 2.86 + (double)g.m * g.n * ksplit * 8.0 / 7.38e6;
@@ -167,16 +170,32 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
     Plan p{FP8GEMM_KERNEL_SCALAR, 0, 1};
     if (selected == FP8GEMM_KERNEL_SCALAR)
         return p;
-    if (selected == FP8GEMM_KERNEL_SKINNY || (selected == FP8GEMM_KERNEL_AUTO && skinny_supports(g) && g.m <= 64)) {
-        if (skinny_supports(g)) {
-            p.family = FP8GEMM_KERNEL_SKINNY;
-            p.ksplit = skinny_ksplit(g);
-            return p;
+    // The decode kernel (M <= 32).  Asked for by name, or with a K split pinned, it runs whenever it can;
+    // under automatic dispatch it has to hold its own against the best tile plan by cost: with a long K
+    // range and many column strips its workgroups go through several copy-wait-multiply passes, and 64x64
+    // tiles with the K range split are faster (measured: 12-14 us against 15-20 us for M = 16 / 32,
+    // N >= 4608, K = 7168).
+    Plan decode{FP8GEMM_KERNEL_SKINNY, 0, 1};
+    double decode_us = -1.0;  // >= 0: the decode kernel is a candidate, at this cost
+    if (selected == FP8GEMM_KERNEL_SKINNY && !skinny_supports(g)) {
+        p.family = -1;
+        return p;
+    }
+    if (skinny_supports(g) && (selected == FP8GEMM_KERNEL_SKINNY || selected == FP8GEMM_KERNEL_AUTO)) {
+        decode.ksplit = skinny_ksplit(g);
+        if (cfg.force_ksplit > 0) {  // every split has to own at least one K block
+            const int nkb = g.k / 128;
+            int ks = cfg.force_ksplit < nkb ? cfg.force_ksplit : nkb;
+            while (ks > 1 && (ks - 1) * ((nkb + ks - 1) / ks) >= nkb)
+                --ks;
+            decode.ksplit = ks;
         }
-        if (selected == FP8GEMM_KERNEL_SKINNY) {
-            p.family = -1;
-            return p;
-        }
+        if (selected == FP8GEMM_KERNEL_SKINNY || cfg.force_variant >= 0 || cfg.force_ksplit > 0 || !tile_supports(g))
+            return decode;
+        // one pass of one round of workgroups, no K split: nothing here is faster (4.3-5.2 us measured)
+        if (decode.ksplit == 1 && skinny_cost(g, 1) <= skinny_cost(g, 0))
+            return decode;
+        decode_us = skinny_cost(g, decode.ksplit);
     }
     if (!tile_supports(g)) {
         if (selected != FP8GEMM_KERNEL_AUTO) {
@@ -215,6 +234,8 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             continue;
         if (v == TILE_256x192_W4 && fv != v)  // one-wave-per-SIMD form: only when asked for
             continue;
+        if (g.m <= 64 && fv < 0 && selected == FP8GEMM_KERNEL_AUTO && v != TILE_64x64)
+            continue;  // a single row of tiles: taller tiles only multiply rows that do not exist
         for (int ks = 1; ks <= MAX_KSPLIT && ks <= nkb; ++ks) {
             if (v == TILE_256x192_W4 && ks != 1)
                 continue;
@@ -228,6 +249,10 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             const int kbs = (nkb + ks - 1) / ks;
             if ((ks - 1) * kbs >= nkb)
                 continue;
+            // a single row of tiles: the fitted constants overrate a split into short K ranges (measured
+            // for M = 16 ... 64: the best split never leaves a workgroup fewer than 8 K blocks)
+            if (g.m <= 64 && fk <= 0 && selected == FP8GEMM_KERNEL_AUTO && ks > 1 && kbs < 8)
+                continue;
             const double cst = tile_cost(g, v, ks);
             if (cst < best) {
                 best = cst;
@@ -237,6 +262,8 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             }
         }
     }
+    if (decode_us >= 0.0 && decode_us <= 0.95 * best)  // measured: at equal estimates the decode kernel is ahead
+        return decode;
     if (best == 1e300) {
         p.family = -1;
         return p;
@@ -307,7 +334,7 @@ hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, hipStre
     case FP8GEMM_KERNEL_SCALAR:
         return launch_scalar(g, stream);
     case FP8GEMM_KERNEL_SKINNY:
-        return launch_skinny(g, partial, stream);
+        return launch_skinny(g, p.ksplit, partial, stream);
     default: {
         if (p.persistent)
             return launch_tile_persistent(g, p.variant, NUM_CU, stream);

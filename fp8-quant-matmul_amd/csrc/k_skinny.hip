@@ -187,22 +187,50 @@ bool skinny_supports(const GemmArgs& g)
            (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
 }
 
-// Split K across workgroups only when the column strips alone cannot occupy the chip.
-int skinny_ksplit(const GemmArgs& g)
+// Microseconds, fitted to measurements with M = 16 and 32, N = 1536 ... 7168, K = 1536 ... 7168 (operands in
+// the caches).  A wave copies and multiplies two K blocks per pass, eight waves per workgroup: up to 16
+// K blocks of a workgroup's range go in one pass, which the 4.4 us cover (launch, one pass, the LDS
+// reduction, the store); every further pass, or further round of 256 workgroups, waits for its copies again
+// and costs in proportion to the workgroups that pull on the memory system together; a K split over
+// workgroups adds the reduction launch and the partial sums.
+double skinny_cost(const GemmArgs& g, int ksplit)
 {
-    const int tiles_n = (g.n + SK_BN - 1) / SK_BN;
+    if (ksplit <= 0)  // the floor: one pass of one round, no K split
+        return 4.4;
+    const int strips = (g.n + SK_BN - 1) / SK_BN;
     const int nkb = g.k / KBLOCK;
-    int ks = 1;
-    while (tiles_n * ks < 192 && ks * 2 <= nkb / 8 && ks < 16)
-        ks *= 2;
-    return ks;
+    const int kbs = (nkb + ksplit - 1) / ksplit;
+    const int passes = ((kbs + 7) / 8 + SK_CHUNK_KB - 1) / SK_CHUNK_KB;
+    const long wgs = (long)strips * ksplit;
+    const long rounds = (wgs + 255) / 256;
+    const double together = wgs < 256 ? (double)wgs : 256.0;
+    return 4.4 + (ksplit > 1 ? 2.7 : 0.0) + (double)(passes * rounds - 1) * 0.028 * together;
 }
 
-hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s)
+// the K split (over workgroups) with the lowest cost; every split owns at least one K block
+int skinny_ksplit(const GemmArgs& g)
+{
+    const int nkb = g.k / KBLOCK;
+    int best = 1;
+    double best_cost = skinny_cost(g, 1);
+    for (int ks = 2; ks <= 8 && ks <= nkb; ++ks) {
+        if ((ks - 1) * ((nkb + ks - 1) / ks) >= nkb)
+            continue;
+        const double c = skinny_cost(g, ks);
+        if (c < best_cost) {
+            best_cost = c;
+            best = ks;
+        }
+    }
+    return best;
+}
+
+hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStream_t s)
 {
     const int tiles_n = (g.n + SK_BN - 1) / SK_BN;
     const int nkb = g.k / KBLOCK;
-    const int ksplit = partial ? skinny_ksplit(g) : 1;
+    if (ksplit < 1 || ksplit > nkb || ksplit > 65535 || (ksplit > 1 && !partial))
+        return hipErrorInvalidValue;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     dim3 grid(tiles_n, ksplit);
     hipError_t e;

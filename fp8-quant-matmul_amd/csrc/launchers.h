@@ -79,7 +79,8 @@ hipError_t launch_splitk_reduce(const GemmArgs& g, int ksplit, const float* part
 // tiny-M streaming kernel (decode shapes)
 bool skinny_supports(const GemmArgs& g);
 int skinny_ksplit(const GemmArgs& g);
-hipError_t launch_skinny(const GemmArgs& g, float* partial, hipStream_t s);
+double skinny_cost(const GemmArgs& g, int ksplit);
+hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStream_t s);
 
 // rows of ld_src elements copied into rows of ld_dst >= ld_src elements, the rest zero (dst
 // 16-byte aligned, ld_dst a multiple of 16 bytes); the m x n corner of a bf16 matrix with

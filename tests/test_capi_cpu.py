@@ -197,6 +197,19 @@ def test_dispatcher_plans(pkg):
     assert pkg.workspace_bytes(33, 100, 128) >= 128 * 48 + 128 * 112 + 48 * 4 + 48 * 112 * 2
     ks = int(pkg.plan(2048, 576, 7168).split("_k")[1])
     assert ks > 1                                          # few tiles, long K: split
+    # decode shapes (M <= 32): the streaming kernel while a workgroup's K range goes in one pass, its K range
+    # split when the strips alone leave CUs idle, 64x64 tiles with a K split when strips AND K are many
+    assert pkg.plan(32, 7168, 2048) == "skinny_k1"
+    assert pkg.plan(16, 1536, 2048) == "skinny_k1"
+    assert pkg.plan(32, 1536, 7168) == "skinny_k4"
+    assert pkg.plan(32, 7168, 7168) == "tile64x64_k4"
+    assert pkg.plan(16, 4608, 7168) == "tile64x64_k7"
+    assert pkg.plan(64, 1536, 7168) == "tile64x64_k7"      # a single row of tiles: never fewer than 8 K blocks per split
+    assert pkg.plan(48, 1536, 1536) == "tile64x64_k1"
+    pkg.select(pkg.KERNEL_SKINNY)
+    pkg.force_config(-1, 3)
+    assert pkg.plan(32, 7168, 2048) == "skinny_k3"         # a pinned K split reaches the decode kernel too
+    pkg.force_config(-1, 0)
     pkg.select(pkg.KERNEL_SCALAR)
     assert pkg.plan(8192, 4608, 7168) == "scalar"
     pkg.select(pkg.KERNEL_SKINNY)

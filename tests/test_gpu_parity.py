@@ -179,6 +179,28 @@ def test_skinny_kernel(pkg, m, n, k):
     _assert_close(got, ref, name)
 
 
+@pytest.mark.parametrize("m,n,k,ksplit", [(32, 1536, 7168, 4), (16, 1040, 2048, 2), (32, 576, 7168, 7),
+                                          (32, 96, 1024, 8), (16, 4608, 1536, 3)])
+def test_skinny_kernel_with_the_k_range_split_over_workgroups(pkg, m, n, k, ksplit):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 950 + n + ksplit)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, ksplit=ksplit)
+    assert name == f"skinny_k{ksplit}", name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+
+
+@pytest.mark.parametrize("m,n,k", [(32, 7168, 7168), (16, 4608, 7168), (32, 1536, 7168), (32, 7168, 4096),
+                                   (48, 1536, 4096), (64, 7168, 2048)])
+def test_decode_shapes_under_automatic_dispatch(pkg, m, n, k):
+    """what the dispatcher picks for small M (decode kernel, its K split, or 64x64 tiles with a K split)"""
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 990 + m + n // 7)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k)
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+
+
 @pytest.mark.parametrize("m,n,k", [(33, 100, 128), (17, 129, 256), (100, 100, 384)])
 def test_scalar_kernel_takes_unaligned_shapes(pkg, m, n, k):
     a, b, sa, sb = oracle.make_inputs(m, n, k, 5 + m)
