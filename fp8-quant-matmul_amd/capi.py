@@ -14,14 +14,17 @@ _LIB = None
 
 KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5)
 DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH = 0, 1, 2
+FLAG_WORKSPACE_ZEROED = 1
+WORKSPACE_HEADER_BYTES = 16384
 
 
 class Options(C.Structure):
     """fp8gemm_options of the header: per-call kernel choice for gemm_ex"""
-    _fields_ = [("kernel", C.c_int), ("tile_variant", C.c_int), ("ksplit", C.c_int), ("persistent", C.c_int)]
+    _fields_ = [("kernel", C.c_int), ("tile_variant", C.c_int), ("ksplit", C.c_int), ("persistent", C.c_int),
+                ("flags", C.c_int)]
 
-    def __init__(self, kernel=KERNEL_AUTO, tile_variant=-1, ksplit=0, persistent=-1):
-        super().__init__(kernel, tile_variant, ksplit, persistent)
+    def __init__(self, kernel=KERNEL_AUTO, tile_variant=-1, ksplit=0, persistent=-1, flags=0):
+        super().__init__(kernel, tile_variant, ksplit, persistent, flags)
 
 
 class Fp8GemmError(RuntimeError):
@@ -92,6 +95,8 @@ def lib():
     L.fp8_block_gemm_set_workspace.argtypes = [vp, sz]
     L.fp8_block_gemm_release.restype = i
     L.fp8_block_gemm_release.argtypes = []
+    L.fp8_block_gemm_workspace_growth.restype = sz
+    L.fp8_block_gemm_workspace_growth.argtypes = [sz, sz]
     L.fp8_convert_f32_to_e4m3fn.restype = i
     L.fp8_convert_f32_to_e4m3fn.argtypes = [vp, vp, sz, vp]
     L.fp8_quantize_a_1x128.restype = i

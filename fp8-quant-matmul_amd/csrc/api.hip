@@ -32,24 +32,53 @@ struct Config {
     int force_variant;  // tile shape, -1 = cost model
     int force_ksplit;   // 0 = cost model
     int persistent;     // -1 / 0 / 1 as above
+    // plans that add K splits inside the kernel may be chosen: the workspace starts with zeroed ticket
+    // words and the device places workgroups on XCDs as those kernels assume (set by run())
+    bool fused_ok = true;
 };
 Config global_config() { return Config{g_selected.load(), g_force_variant.load(), g_force_ksplit.load(), g_persistent.load()}; }
 constexpr int MAX_KSPLIT = 16;
 
 // device memory a call may use beyond its operands: fp32 partial sums of plans that split K, padded
 // copies of operands off the 16-byte grid
+// The first WS_HEADER bytes hold the arrival tickets of the kernels that add their K splits
+// themselves (zero before the first call and after every call); plans keep their data behind it.
 struct Workspace {
     float* ptr;
     size_t bytes;
+    bool zeroed;  // the header was zero-filled when the buffer was taken on and only this library wrote to it since
 };
+constexpr size_t WS_HEADER = (size_t)DECODE_TICKET_WORDS * sizeof(unsigned int);
+inline float* ws_data(const Workspace& w) { return w.ptr ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(w.ptr) + WS_HEADER) : nullptr; }
+inline unsigned int* ws_tickets(const Workspace& w) { return reinterpret_cast<unsigned int*>(w.ptr); }
 
 std::mutex g_ws_mutex;
 float* g_ws_own = nullptr;       // library-owned workspace
 size_t g_ws_own_bytes = 0;
-std::vector<void*> g_ws_retired; // outgrown library-owned buffers: kernels in flight and captured graphs may
-                                 // still use them, so they live until fp8_block_gemm_release()
+bool g_ws_own_captured = false;  // handed out to a call whose stream was being captured: a graph holds its address
+hipStream_t g_ws_last_stream = nullptr;  // stream of the last call that was given the library-owned workspace
+// Outgrown library-owned buffers.  Kernels of earlier calls may still use one: it is freed by a later
+// growth once the event recorded behind its last use has completed.  One that a captured graph may hold
+// (pinned) lives until fp8_block_gemm_release().
+struct Retired {
+    void* ptr;
+    hipEvent_t done;  // nullptr when pinned
+    bool pinned;
+};
+std::vector<Retired> g_ws_retired;
 float* g_ws_user = nullptr;      // caller-supplied workspace
 size_t g_ws_user_bytes = 0;
+bool g_ws_user_zeroed = false;
+
+// Size the library-owned workspace grows to when a call needs `need` bytes and `have` are there: at
+// least double, so that the buffers retired on the way never add up to more than the live one.
+size_t growth_target(size_t have, size_t need)
+{
+    if (need <= have)
+        return have;
+    const size_t twice = have > (SIZE_MAX >> 1) ? SIZE_MAX : 2 * have;
+    return need > twice ? need : twice;
+}
 
 struct Plan {
     int family;   // FP8GEMM_KERNEL_*
@@ -57,6 +86,7 @@ struct Plan {
     int ksplit;
     bool persistent = false;  // tile families, ksplit == 1: workgroups walk through the tiles
     bool padded = false;      // the plan is for the problem with m and n rounded up to 16 (run_padded)
+    bool wide = false;        // decode family: 128-column strips, K splits added inside the kernel (k_decode.hip)
 };
 
 // Shapes or addresses the MFMA kernels cannot take (m or n not a multiple of 16, a base not
@@ -170,32 +200,72 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
     Plan p{FP8GEMM_KERNEL_SCALAR, 0, 1};
     if (selected == FP8GEMM_KERNEL_SCALAR)
         return p;
-    // The decode kernel (M <= 32).  Asked for by name, or with a K split pinned, it runs whenever it can;
-    // under automatic dispatch it has to hold its own against the best tile plan by cost: with a long K
-    // range and many column strips its workgroups go through several copy-wait-multiply passes, and 64x64
-    // tiles with the K range split are faster (measured: 12-14 us against 15-20 us for M = 16 / 32,
+    // The decode kernels (M <= 32): narrow strips (k_skinny.hip) or wide strips whose K splits are added
+    // inside the kernel (k_decode.hip), whichever the cost model prefers; with the family asked for by name,
+    // tile_variant 0 / 1 pins the narrow / wide form.  Under automatic dispatch the family has to hold its own
+    // against the best tile plan by cost: with a long K range and many column strips 64x64 tiles with the K
+    // range split are faster than the narrow kernel (measured: 12-14 us against 15-20 us for M = 16 / 32,
     // N >= 4608, K = 7168).
     Plan decode{FP8GEMM_KERNEL_SKINNY, 0, 1};
-    double decode_us = -1.0;  // >= 0: the decode kernel is a candidate, at this cost
-    if (selected == FP8GEMM_KERNEL_SKINNY && !skinny_supports(g)) {
+    double decode_us = -1.0;  // >= 0: the decode family is a candidate, at this cost
+    const bool narrow_ok = skinny_supports(g), wide_ok = decode_strip_supports(g);
+    if (selected == FP8GEMM_KERNEL_SKINNY && !narrow_ok && !wide_ok) {
         p.family = -1;
         return p;
     }
-    if (skinny_supports(g) && (selected == FP8GEMM_KERNEL_SKINNY || selected == FP8GEMM_KERNEL_AUTO)) {
-        decode.ksplit = skinny_ksplit(g);
+    if ((narrow_ok || wide_ok) && (selected == FP8GEMM_KERNEL_SKINNY || selected == FP8GEMM_KERNEL_AUTO)) {
+        const int nkb = g.k / 128;
+        const bool by_name = selected == FP8GEMM_KERNEL_SKINNY;
+        auto valid_split = [&](int ks) { return ks >= 1 && ks <= nkb && (ks - 1) * ((nkb + ks - 1) / ks) < nkb; };
+        int forced_ks = 0;
         if (cfg.force_ksplit > 0) {  // every split has to own at least one K block
-            const int nkb = g.k / 128;
-            int ks = cfg.force_ksplit < nkb ? cfg.force_ksplit : nkb;
-            while (ks > 1 && (ks - 1) * ((nkb + ks - 1) / ks) >= nkb)
-                --ks;
-            decode.ksplit = ks;
+            forced_ks = cfg.force_ksplit < nkb ? cfg.force_ksplit : nkb;
+            while (!valid_split(forced_ks))
+                --forced_ks;
         }
-        if (selected == FP8GEMM_KERNEL_SKINNY || cfg.force_variant >= 0 || cfg.force_ksplit > 0 || !tile_supports(g))
-            return decode;
-        // one pass of one round of workgroups, no K split: nothing here is faster (4.3-5.2 us measured)
-        if (decode.ksplit == 1 && skinny_cost(g, 1) <= skinny_cost(g, 0))
-            return decode;
-        decode_us = skinny_cost(g, decode.ksplit);
+        double narrow_us = 1e300, wide_us = 1e300;
+        Plan narrow = decode, wide = decode;
+        wide.wide = true;
+        if (narrow_ok && !(by_name && cfg.force_variant == 1)) {
+            narrow.ksplit = forced_ks ? forced_ks : skinny_ksplit(g);
+            narrow_us = skinny_cost(g, narrow.ksplit);
+        }
+        if (wide_ok && (by_name ? cfg.force_variant != 0 : cfg.force_variant < 0)) {
+            // without the in-kernel reduction (no zeroed tickets, or workgroup placement not confirmed) only
+            // the unsplit form exists
+            const int hi = cfg.fused_ok ? (nkb < MAX_KSPLIT ? nkb : MAX_KSPLIT) : 1;
+            for (int ks = 1; ks <= hi; ++ks) {
+                if (!valid_split(ks) || (forced_ks && ks != forced_ks))
+                    continue;
+                const double cst = decode_strip_cost(g, ks);
+                if (cst < wide_us) {
+                    wide_us = cst;
+                    wide.ksplit = ks;
+                }
+            }
+        }
+        // Decode weights come from HBM (a model's layers do not fit the caches): there the wide strips are
+        // ahead of the narrow ones and of every tile plan on all 40 shapes measured (M = 16, 32; N = 1536 ...
+        // 16384; K = 1536 ... 7168: 6.0-27 us against 7.3-60 us), although the narrow kernel is 1-2 us faster
+        // on short K when B happens to sit in the Infinity Cache.  They need the in-kernel reduction.
+        if (!by_name && cfg.force_variant < 0 && cfg.force_ksplit <= 0 && wide_us < 1e300 && cfg.fused_ok)
+            return wide;
+        if (!by_name && !cfg.fused_ok)
+            wide_us = 1e300;  // unsplit wide strips leave most CUs idle: the narrow kernel and the tile plans compete
+        if (narrow_us == 1e300 && wide_us == 1e300) {
+            if (by_name) {
+                p.family = -1;
+                return p;
+            }
+        } else {
+            decode = wide_us < narrow_us ? wide : narrow;
+            decode_us = wide_us < narrow_us ? wide_us : narrow_us;
+            if (by_name || cfg.force_variant >= 0 || cfg.force_ksplit > 0 || !tile_supports(g))
+                return decode;
+            // one pass of one round of workgroups: nothing here is faster
+            if (decode_us <= skinny_cost(g, 0))
+                return decode;
+        }
     }
     if (!tile_supports(g)) {
         if (selected != FP8GEMM_KERNEL_AUTO) {
@@ -275,45 +345,89 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
 }
 
 // The process-wide workspace for a call on `stream` that needs `bytes`: the caller-supplied one, else
-// the library-owned one, grown on demand.  Growing allocates, which a stream under capture does not
-// allow (and which would leave the graph with a buffer it was not recorded with): such a call gets
-// FP8GEMM_E_WORKSPACE and the capture stays valid.  Nothing here waits for the device: an outgrown
-// buffer is retired, not freed.
+// the library-owned one, grown on demand (growth_target).  Growing allocates, which a stream under
+// capture does not allow (and which would leave the graph with a buffer it was not recorded with): such
+// a call gets FP8GEMM_E_WORKSPACE and the capture stays valid.  An outgrown buffer is retired, not
+// freed on the spot: kernels in flight may still use it.
 int acquire_workspace(size_t bytes, hipStream_t stream, Workspace* out)
 {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     if (g_ws_user) {
         if (g_ws_user_bytes < bytes)
             return FP8GEMM_E_WORKSPACE;
-        *out = Workspace{g_ws_user, g_ws_user_bytes};
+        *out = Workspace{g_ws_user, g_ws_user_bytes, g_ws_user_zeroed};
         return FP8GEMM_OK;
     }
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    hipError_t e = hipStreamIsCapturing(stream, &status);
+    if (e != hipSuccess)
+        return (int)e;
+    const bool capturing = status != hipStreamCaptureStatusNone;
     if (g_ws_own_bytes < bytes) {
-        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-        hipError_t e = hipStreamIsCapturing(stream, &status);
-        if (e != hipSuccess)
-            return (int)e;
-        if (status != hipStreamCaptureStatusNone)
+        if (capturing)
             return FP8GEMM_E_WORKSPACE;
+        // retired buffers whose last use has completed go back to the allocator now
+        for (size_t i = 0; i < g_ws_retired.size();) {
+            Retired& r = g_ws_retired[i];
+            if (!r.pinned && hipEventQuery(r.done) == hipSuccess) {
+                (void)hipEventDestroy(r.done);
+                (void)hipFree(r.ptr);
+                g_ws_retired.erase(g_ws_retired.begin() + (long)i);
+            } else {
+                ++i;
+            }
+        }
+        (void)hipGetLastError();  // hipEventQuery reports "not ready" as an error
+        size_t want = growth_target(g_ws_own_bytes, bytes);
         void* p = nullptr;
-        e = hipMalloc(&p, bytes);
+        e = hipMalloc(&p, want);
+        if (e != hipSuccess && want > bytes) {
+            (void)hipGetLastError();
+            want = bytes;
+            e = hipMalloc(&p, want);
+        }
         if (e != hipSuccess)
             return (int)e;
-        if (g_ws_own)
-            g_ws_retired.push_back(g_ws_own);
+        e = hipMemset(p, 0, WS_HEADER);  // the ticket words (bytes >= WS_HEADER whenever a plan needs a workspace)
+        if (e != hipSuccess) {
+            (void)hipFree(p);
+            return (int)e;
+        }
+        if (g_ws_own) {
+            Retired r{g_ws_own, nullptr, g_ws_own_captured};
+            if (!r.pinned) {
+                if (hipEventCreateWithFlags(&r.done, hipEventDisableTiming) != hipSuccess ||
+                    hipEventRecord(r.done, g_ws_last_stream) != hipSuccess) {
+                    (void)hipGetLastError();
+                    if (r.done)
+                        (void)hipEventDestroy(r.done);
+                    r.done = nullptr;
+                    r.pinned = true;  // no way to tell when its last use ends: kept until release
+                }
+            }
+            g_ws_retired.push_back(r);
+        }
         g_ws_own = static_cast<float*>(p);
-        g_ws_own_bytes = bytes;
+        g_ws_own_bytes = want;
+        g_ws_own_captured = false;
     }
-    *out = Workspace{g_ws_own, g_ws_own_bytes};
+    g_ws_own_captured = g_ws_own_captured || capturing;
+    g_ws_last_stream = stream;
+    *out = Workspace{g_ws_own, g_ws_own_bytes, true};
     return FP8GEMM_OK;
 }
 
+// bytes of partial sums a plan keeps behind the workspace header
 size_t plan_workspace_bytes(const GemmArgs& g, const Plan& p)
 {
     if (p.ksplit <= 1)
         return 0;
+    if (p.family == FP8GEMM_KERNEL_SKINNY && p.wide)
+        return decode_strip_partial_bytes(g, p.ksplit);
     return (size_t)p.ksplit * g.m * g.n * sizeof(float);
 }
+// a workspace that holds `data` bytes of a plan: nothing, or the header and the data
+inline size_t with_header(size_t data) { return data ? data + WS_HEADER : 0; }
 
 void plan_name(const Plan& p, char* out, size_t cap)
 {
@@ -321,19 +435,22 @@ void plan_name(const Plan& p, char* out, size_t cap)
     if (p.family == FP8GEMM_KERNEL_SCALAR)
         snprintf(out, cap, "scalar");
     else if (p.family == FP8GEMM_KERNEL_SKINNY)
-        snprintf(out, cap, "%sskinny_k%d", pre, p.ksplit);
+        snprintf(out, cap, p.wide ? "%sdecode128_k%d" : "%sskinny_k%d", pre, p.ksplit);
     else
         snprintf(out, cap, "%s%s_k%d%s", pre, tile_variant_name(p.variant), p.ksplit,
                  p.persistent ? "_persistent" : "");
 }
 
-// the kernels of a plan on operands they can take; `partial` holds plan_workspace_bytes
-hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, hipStream_t stream)
+// the kernels of a plan on operands they can take; `partial` holds plan_workspace_bytes, `tickets` the
+// zeroed words of the workspace header (plans that add their K splits inside the kernel)
+hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, unsigned int* tickets, hipStream_t stream)
 {
     switch (p.family) {
     case FP8GEMM_KERNEL_SCALAR:
         return launch_scalar(g, stream);
     case FP8GEMM_KERNEL_SKINNY:
+        if (p.wide)
+            return launch_decode_strips(g, p.ksplit, partial, tickets, stream);
         return launch_skinny(g, p.ksplit, partial, stream);
     default: {
         if (p.persistent)
@@ -354,7 +471,7 @@ size_t padded_bytes(const GemmArgs& g, const Plan& p)
     gp.m = (g.m + 15) & ~15;
     gp.n = (g.n + 15) & ~15;
     const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK;
-    return pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows).total;
+    return with_header(pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows).total);
 }
 
 int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t stream)
@@ -369,9 +486,9 @@ int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t
         gp.m = g.m;
         gp.lda = m16;
     }
-    if (!w.ptr || w.bytes < L.total)
+    if (!w.ptr || w.bytes < with_header(L.total))
         return FP8GEMM_E_WORKSPACE;
-    uint8_t* base = reinterpret_cast<uint8_t*>(w.ptr);
+    uint8_t* base = reinterpret_cast<uint8_t*>(ws_data(w));
     const int nkb = g.k / 128;
     hipError_t e = hipSuccess;
     if (L.a) {
@@ -390,27 +507,53 @@ int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t
     if (L.c)
         gp.c = reinterpret_cast<uint16_t*>(base + L.off_c);
     if (e == hipSuccess)
-        e = launch_plan(gp, p, reinterpret_cast<float*>(base + L.off_partial), stream);
+        e = launch_plan(gp, p, reinterpret_cast<float*>(base + L.off_partial), ws_tickets(w), stream);
     if (e == hipSuccess && L.c)
         e = launch_crop_bf16(gp.c, g.c, g.m, g.n, gp.n, stream);
     return (int)e;
 }
 
+// Whether plans that add their K splits inside the kernel may run for a call on `stream`: the device
+// must place workgroups on XCDs as those kernels assume.  The first call on a device finds out with a
+// probe grid that it waits for; while `stream` is being captured nothing is probed and an unknown
+// placement counts as "no".
+bool placement_ok(hipStream_t stream)
+{
+    int known = xcd_placement_confirmed(false);
+    if (known >= 0)
+        return known == 1;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone)
+        return false;
+    return xcd_placement_confirmed(true) == 1;
+}
+
 // One GEMM.  explicit_ws = the caller's per-call workspace (its bytes may be 0 / its pointer NULL when the
 // plan needs none); nullptr = the process-wide workspace.
 int run(const void* a, const void* b, const float* as, const float* bs, void* c, int m, int n, int k,
-        hipStream_t stream, const Config& cfg, const Workspace* explicit_ws)
+        hipStream_t stream, Config cfg, const Workspace* explicit_ws)
 {
     int v = validate(a, b, as, bs, c, m, n, k);
     if (v != FP8GEMM_OK)
         return v;
     GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), as, bs,
                static_cast<uint16_t*>(c), m, n, k};
+    // in-kernel K-split reduction: zeroed ticket words (every process-wide workspace has them; a per-call
+    // one when the caller says so) and a confirmed workgroup placement
+    cfg.fused_ok = cfg.fused_ok && (!explicit_ws || explicit_ws->zeroed);
+    if (cfg.fused_ok) {
+        Config probe = cfg;
+        probe.fused_ok = false;
+        const Plan with = make_plan(g, cfg), without = make_plan(g, probe);
+        const bool differs = with.family != without.family || with.ksplit != without.ksplit || with.wide != without.wide;
+        if (differs && !placement_ok(stream))
+            cfg.fused_ok = false;
+    }
     const Plan p = make_plan(g, cfg);
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
-    const size_t need = p.padded ? padded_bytes(g, p) : plan_workspace_bytes(g, p);
-    Workspace w{nullptr, 0};
+    const size_t need = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p));
+    Workspace w{nullptr, 0, false};
     if (need) {
         if (explicit_ws) {
             if (!explicit_ws->ptr || explicit_ws->bytes < need ||
@@ -423,7 +566,7 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
                 return rc;
         }
     }
-    const int rc = p.padded ? run_padded(g, p, w, stream) : (int)launch_plan(g, p, w.ptr, stream);
+    const int rc = p.padded ? run_padded(g, p, w, stream) : (int)launch_plan(g, p, ws_data(w), ws_tickets(w), stream);
     if (rc == FP8GEMM_OK) {
         plan_name(p, t_name_buf, sizeof(t_name_buf));
         t_last_kernel = t_name_buf;
@@ -517,13 +660,13 @@ int run_grouped_padded(const GroupTable& tab, int n, int k, hipStream_t s)
         off_c[g] = off;
         off += pad_c ? round256((size_t)m16 * n16 * 2) : 0;
     }
-    Workspace w{nullptr, 0};
-    const int wrc = acquire_workspace(off, s, &w);
+    Workspace w{nullptr, 0, false};
+    const int wrc = acquire_workspace(with_header(off), s, &w);
     if (wrc == FP8GEMM_E_WORKSPACE)
         return GROUPED_NOT_APPLICABLE;  // a caller-supplied workspace sized for single problems: one by one
     if (wrc != FP8GEMM_OK)
         return wrc;
-    uint8_t* base = reinterpret_cast<uint8_t*>(w.ptr);
+    uint8_t* base = reinterpret_cast<uint8_t*>(ws_data(w));
     GroupTable pt;
     RepackTable ta, tas, tb, tc;
     pt.groups = ta.groups = tas.groups = tb.groups = tc.groups = tab.groups;
@@ -570,7 +713,7 @@ Config config_from_options(const fp8gemm_options* opt, int* rc)
         return Config{FP8GEMM_KERNEL_AUTO, -1, 0, -1};
     if (opt->kernel < FP8GEMM_KERNEL_AUTO || opt->kernel > FP8GEMM_KERNEL_SKINNY ||
         opt->tile_variant >= TILE_VARIANT_COUNT || opt->ksplit < 0 || opt->ksplit > MAX_KSPLIT ||
-        opt->persistent < -1 || opt->persistent > 1)
+        opt->persistent < -1 || opt->persistent > 1 || (opt->flags & ~FP8GEMM_FLAG_WORKSPACE_ZEROED) != 0)
         *rc = FP8GEMM_E_KERNEL;
     return Config{opt->kernel, opt->tile_variant < 0 ? -1 : opt->tile_variant, opt->ksplit, opt->persistent};
 }
@@ -590,7 +733,8 @@ size_t workspace_bytes_for(int m, int n, int k, const Config& cfg, bool any_alig
     gp.n = (n + 15) & ~15;
     size_t need = 0;
     if (p.family >= 0)
-        need = p.padded ? pad_layout(g, plan_workspace_bytes(gp, p), true, false).total : plan_workspace_bytes(g, p);
+        need = with_header(p.padded ? pad_layout(g, plan_workspace_bytes(gp, p), true, false).total
+                                    : plan_workspace_bytes(g, p));
     if (any_alignment && !(p.family >= 0 && p.padded)) {
         // the same shape with an operand off a 16-byte boundary: the plan of the padded shape on copies
         const long long lim = 0x7FFFFFFFll;
@@ -598,7 +742,7 @@ size_t workspace_bytes_for(int m, int n, int k, const Config& cfg, bool any_alig
             cfg.selected != FP8GEMM_KERNEL_SCALAR) {
             const Plan pp = make_plan(gp, cfg);
             if (pp.family >= 0 && pp.family != FP8GEMM_KERNEL_SCALAR) {
-                const size_t all = pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total;
+                const size_t all = with_header(pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total);
                 need = all > need ? all : need;
             }
         }
@@ -630,7 +774,8 @@ int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const 
     const Config cfg = config_from_options(options, &rc);
     if (rc != FP8GEMM_OK)
         return rc;
-    const Workspace w{static_cast<float*>(workspace), workspace ? workspace_bytes : 0};
+    const bool zeroed = options && (options->flags & FP8GEMM_FLAG_WORKSPACE_ZEROED) != 0;
+    const Workspace w{static_cast<float*>(workspace), workspace ? workspace_bytes : 0, zeroed};
     return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), cfg, &w);
 }
 
@@ -651,17 +796,25 @@ int fp8_block_gemm_noalloc(const void* a, const void* b, const float* a_scale, c
     const Config cfg = global_config();
     const GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), a_scale, b_scale,
                      static_cast<uint16_t*>(c), m, n, k};
-    const Plan p = make_plan(g, cfg);
-    if (p.family < 0)
-        return FP8GEMM_E_KERNEL;
-    const size_t need = p.padded ? padded_bytes(g, p) : plan_workspace_bytes(g, p);
+    // the largest need among the plans run() may settle on (with and without the in-kernel reduction)
+    size_t need = 0;
+    for (int fused = 0; fused < 2; ++fused) {
+        Config probe = cfg;
+        probe.fused_ok = fused != 0;
+        const Plan p = make_plan(g, probe);
+        if (p.family < 0)
+            return FP8GEMM_E_KERNEL;
+        const size_t bytes = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p));
+        need = bytes > need ? bytes : need;
+    }
     if (need > (size_t)FP8GEMM_NOALLOC_MAX_BYTES)
         return FP8GEMM_E_WORKSPACE;
     void* ptr = nullptr;
     const int rc = scratch_for_current_device(&ptr);
     if (rc != FP8GEMM_OK)
         return rc;
-    const Workspace w{static_cast<float*>(ptr), (size_t)FP8GEMM_NOALLOC_MAX_BYTES};
+    // the array starts out zero and every kernel that uses the ticket words leaves them zero
+    const Workspace w{static_cast<float*>(ptr), (size_t)FP8GEMM_NOALLOC_MAX_BYTES, true};
     return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), cfg, &w);
 }
 
@@ -811,6 +964,11 @@ size_t fp8_block_gemm_grouped_workspace_bytes(int groups, const int* m, int n, i
         const size_t m16 = ((size_t)m[g] + 15) & ~(size_t)15;
         total += round256((size_t)k * m16) + round256(nkb * m16 * sizeof(float)) + round256((size_t)k * n16) +
                  round256(m16 * n16 * 2);
+    }
+    total = with_header(total);
+    for (int g = 0; g < groups; ++g) {
+        if (m[g] <= 0)
+            continue;
         const size_t single = workspace_bytes_for(m[g], n, k, global_config(), true);
         total = total > single ? total : single;
     }
@@ -821,9 +979,19 @@ int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)
 {
     if (device_ptr && (reinterpret_cast<uintptr_t>(device_ptr) % 256) != 0)
         return FP8GEMM_E_WORKSPACE;
+    // the ticket words at its start are zero-filled here (the call waits for that fill); a buffer too
+    // small to hold them can serve no plan anyway
+    bool zeroed = false;
+    if (device_ptr && bytes >= WS_HEADER) {
+        const hipError_t e = hipMemset(device_ptr, 0, WS_HEADER);
+        if (e != hipSuccess)
+            return (int)e;
+        zeroed = true;
+    }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     g_ws_user = static_cast<float*>(device_ptr);
     g_ws_user_bytes = device_ptr ? bytes : 0;
+    g_ws_user_zeroed = zeroed;
     return FP8GEMM_OK;
 }
 
@@ -836,11 +1004,14 @@ int fp8_block_gemm_release(void)
     if (e != hipSuccess)
         return (int)e;
     hipError_t first = hipSuccess;
-    for (void* p : g_ws_retired) {
-        e = hipFree(p);
+    for (Retired& r : g_ws_retired) {
+        if (r.done)
+            (void)hipEventDestroy(r.done);
+        e = hipFree(r.ptr);
         first = first == hipSuccess ? e : first;
     }
     g_ws_retired.clear();
+    g_ws_own_captured = false;
     if (g_ws_own) {
         e = hipFree(g_ws_own);
         first = first == hipSuccess ? e : first;
@@ -911,6 +1082,8 @@ const char* fp8_block_gemm_error_string(int code)
     return "unknown error code";
 }
 
-int fp8_block_gemm_abi_version(void) { return 3; }
+size_t fp8_block_gemm_workspace_growth(size_t have, size_t need) { return growth_target(have, need); }
+
+int fp8_block_gemm_abi_version(void) { return 4; }
 
 }  // extern "C"

@@ -58,7 +58,7 @@ extern "C" int fp8_gemm_host(unsigned short* c, const float* a, const float* b, 
     const float* das = static_cast<const float*>(d_as.p);
     const float* dbs = static_cast<const float*>(d_bs.p);
     // per-call options and a workspace of this call's own: no process-wide switch is touched
-    fp8gemm_options opt{FP8GEMM_KERNEL_AUTO, -1, 0, -1};
+    fp8gemm_options opt{FP8GEMM_KERNEL_AUTO, -1, 0, -1, 0};
     if (option == 2)
         opt.kernel = FP8GEMM_KERNEL_SCALAR;
     else if (option >= 100 && option <= 100 + FP8GEMM_KERNEL_SKINNY)

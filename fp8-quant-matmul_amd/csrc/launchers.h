@@ -82,6 +82,20 @@ int skinny_ksplit(const GemmArgs& g);
 double skinny_cost(const GemmArgs& g, int ksplit);
 hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStream_t s);
 
+// wide-strip decode kernel (M <= 32): 128-column strips, the K splits of a strip added inside the
+// kernel.  `partial` holds decode_strip_partial_bytes; `tickets` = DECODE_TICKET_WORDS words that are
+// zero before the launch and zero again after it.  ksplit > 1 needs xcd_placement_confirmed().
+constexpr int DECODE_TICKET_WORDS = 4096;
+constexpr int DECODE_MAX_KSPLIT = 16;
+bool decode_strip_supports(const GemmArgs& g);
+size_t decode_strip_partial_bytes(const GemmArgs& g, int ksplit);
+double decode_strip_cost(const GemmArgs& g, int ksplit);
+hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* partial, unsigned int* tickets, hipStream_t s);
+// 1 = workgroups whose linear ids agree modulo 8 share an XCD on the current device (looked at once
+// per device with a probe grid, which the first call waits for: not under stream capture),
+// 0 = they do not, or it could not be looked at; -1 = not looked at yet and may_probe is false
+int xcd_placement_confirmed(bool may_probe);
+
 // rows of ld_src elements copied into rows of ld_dst >= ld_src elements, the rest zero (dst
 // 16-byte aligned, ld_dst a multiple of 16 bytes); the m x n corner of a bf16 matrix with
 // ld_src elements per row copied into a dense one

@@ -93,7 +93,9 @@ int fp8_block_gemm_select(int kernel_id);
 /* Pin the MFMA tile kernels to one workgroup tile (0 = 256x192, 1 = 256x128, 2 = 128x128,
  * 3 = 128x192, 4 = 64x64 rows x columns of C, 5 = 256x192 with one wave per SIMD (persistent
  * form only, never chosen automatically); -1 = choose by cost model) and one K-split count
- * (0 = choose, at most 16; more returns FP8GEMM_E_KERNEL).  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
+ * (0 = choose, at most 16; more returns FP8GEMM_E_KERNEL).  With FP8GEMM_KERNEL_SKINNY selected the
+ * first argument picks the decode kernel instead: 0 = 32-column strips, 1 = 128-column strips whose K
+ * splits are added inside the kernel, -1 = by cost.  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
  * (/root/reference/mn_large.hip:1-8). */
 int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 
@@ -131,7 +133,16 @@ typedef struct fp8gemm_options {
     int tile_variant; /* as fp8_block_gemm_force_config; -1 = cost model */
     int ksplit;       /* 0 = cost model, else 1..16 */
     int persistent;   /* as fp8_block_gemm_set_persistent */
+    int flags;        /* FP8GEMM_FLAG_* or 0 */
 } fp8gemm_options;
+/* The first FP8GEMM_WORKSPACE_HEADER_BYTES of the workspace handed to this call were zero-filled by the
+ * caller before the first call that used this workspace, and nothing but this library has written to the
+ * workspace since.  The library keeps arrival tickets there (zero again after every call) for the plans
+ * that add the K splits of a tile or strip inside the GEMM kernel instead of launching a reduction kernel
+ * ("decode128_kN", "..._kNf"); without the flag a per-call workspace only gets the two-kernel plans.
+ * The process-wide workspace and fp8_block_gemm_noalloc's array always have zeroed tickets. */
+#define FP8GEMM_FLAG_WORKSPACE_ZEROED 1
+#define FP8GEMM_WORKSPACE_HEADER_BYTES 16384
 int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
                       int m, int n, int k, const fp8gemm_options* options, void* workspace,
                       size_t workspace_bytes, void* stream);
@@ -191,6 +202,12 @@ size_t fp8_block_gemm_workspace_bytes(int m, int n, int k);
 size_t fp8_block_gemm_grouped_workspace_bytes(int groups, const int* m, int n, int k);
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes);
 int fp8_block_gemm_release(void);
+/* Growth policy of the library-owned workspace: the size it is (re)allocated with when a call needs
+ * `need` bytes and it holds `have` (at least twice `have`, so that outgrown buffers never add up to more
+ * than the live one).  An outgrown buffer is freed by a later growth once the work that last used it has
+ * completed; one that was handed to a call under stream capture is kept until fp8_block_gemm_release.
+ * Touches no device.  No counterpart in the reference. */
+size_t fp8_block_gemm_workspace_growth(size_t have, size_t need);
 
 /* fp32 -> fp8 e4m3fn, round to nearest even, saturating to +-448; count elements; `in` 16-byte and
  * `out` 4-byte aligned (FP8GEMM_E_ALIGN otherwise).

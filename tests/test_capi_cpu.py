@@ -14,7 +14,7 @@ def test_library_exports_every_declared_symbol(pkg):
     assert len(names) >= 22
     for name in names:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
-    assert L.fp8_block_gemm_abi_version() == 3
+    assert L.fp8_block_gemm_abi_version() == 4
 
 
 def test_argument_validation_happens_before_any_device_call(pkg):
@@ -99,10 +99,11 @@ def test_workspace_contract(pkg):
     assert pkg.workspace_bytes(64, 64, 128) == 0                     # one K block: nothing to split
     assert pkg.workspace_bytes(8192, 4608, 7168) == 0                # plan does not split K
     assert pkg.plan(1024, 512, 7168) == "tile64x64_k2"
-    assert pkg.workspace_bytes(1024, 512, 7168) == 2 * 1024 * 512 * 4
+    H = pkg.WORKSPACE_HEADER_BYTES                                   # ticket words ahead of every plan's data
+    assert pkg.workspace_bytes(1024, 512, 7168) == H + 2 * 1024 * 512 * 4
     assert L.fp8_block_gemm_force_config(2, 8) == 0                  # follows a forced configuration
     try:
-        assert pkg.workspace_bytes(256, 256, 1024) == 8 * 256 * 256 * 4
+        assert pkg.workspace_bytes(256, 256, 1024) == H + 8 * 256 * 256 * 4
     finally:
         assert L.fp8_block_gemm_force_config(-1, 0) == 0
     assert L.fp8_block_gemm_set_workspace(4096 + 8, 1 << 20) == -4   # misaligned
@@ -123,7 +124,8 @@ def test_per_call_entry_point_validates_and_never_allocates(pkg):
         assert pkg.workspace_bytes_ex(256, 256, 1024, bad) == 0
     split = O(kernel=pkg.KERNEL_SPLITK, tile_variant=2, ksplit=4)
     need = pkg.workspace_bytes_ex(256, 256, 1024, split)
-    assert need == 4 * 256 * 256 * 4
+    assert need == pkg.WORKSPACE_HEADER_BYTES + 4 * 256 * 256 * 4
+    assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(O(flags=2)), None, 0, None) == -3   # unknown flag
     # a plan that needs a workspace and is not given one (or too little, or a misaligned one)
     assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(split), None, 0, None) == -4
     assert L.fp8_block_gemm_ex(p, p, p, p, p, 256, 256, 1024, C.byref(split), p, need - 1, None) == -4
@@ -134,7 +136,7 @@ def test_per_call_entry_point_validates_and_never_allocates(pkg):
     pkg.force_config(1, 4)
     try:
         assert pkg.workspace_bytes_ex(1024, 512, 2048) == pkg.workspace_bytes_ex(1024, 512, 2048, O())
-        assert pkg.workspace_bytes(1024, 512, 2048) == 4 * 1024 * 512 * 4
+        assert pkg.workspace_bytes(1024, 512, 2048) == pkg.WORKSPACE_HEADER_BYTES + 4 * 1024 * 512 * 4
     finally:
         pkg.force_config(-1, 0)
 
@@ -190,25 +192,30 @@ def test_dispatcher_plans(pkg):
     pkg.force_config(-1, 0)
     assert pkg.plan(8192, 4608, 7168).startswith("tile")
     assert "_k1" in pkg.plan(8192, 4608, 7168)
-    assert pkg.plan(32, 7168, 2048).startswith("skinny")
+    assert pkg.plan(32, 7168, 2048).startswith("decode128")
     assert pkg.plan(33, 100, 128).startswith("padded_")   # rows not 16-byte aligned: padded copies
     assert pkg.plan(8191, 4607, 7168) == "padded_" + pkg.plan(8192, 4608, 7168)
     assert pkg.plan(16777215, 16, 128) == "scalar"         # padding would pass the operand size limit
     assert pkg.workspace_bytes(33, 100, 128) >= 128 * 48 + 128 * 112 + 48 * 4 + 48 * 112 * 2
     ks = int(pkg.plan(2048, 576, 7168).split("_k")[1])
     assert ks > 1                                          # few tiles, long K: split
-    # decode shapes (M <= 32): the streaming kernel while a workgroup's K range goes in one pass, its K range
-    # split when the strips alone leave CUs idle, 64x64 tiles with a K split when strips AND K are many
-    assert pkg.plan(32, 7168, 2048) == "skinny_k1"
-    assert pkg.plan(16, 1536, 2048) == "skinny_k1"
-    assert pkg.plan(32, 1536, 7168) == "skinny_k4"
-    assert pkg.plan(32, 7168, 7168) == "tile64x64_k4"
-    assert pkg.plan(16, 4608, 7168) == "tile64x64_k7"
+    # decode shapes (M <= 32): 128-column strips with the K range split so that one round of workgroups
+    # (at most 256) streams B, the splits added inside the kernel
+    assert pkg.plan(32, 7168, 2048) == "decode128_k4"      # 56 strips x 4
+    assert pkg.plan(16, 1536, 2048) == "decode128_k4"
+    assert pkg.plan(32, 16384, 7168) == "decode128_k2"     # 128 strips x 2
+    assert pkg.plan(32, 128, 128) == "decode128_k1"        # one K block: nothing to split
+    assert pkg.workspace_bytes(32, 7168, 2048) == pkg.WORKSPACE_HEADER_BYTES + 56 * 4 * 16384
     assert pkg.plan(64, 1536, 7168) == "tile64x64_k7"      # a single row of tiles: never fewer than 8 K blocks per split
     assert pkg.plan(48, 1536, 1536) == "tile64x64_k1"
     pkg.select(pkg.KERNEL_SKINNY)
     pkg.force_config(-1, 3)
-    assert pkg.plan(32, 7168, 2048) == "skinny_k3"         # a pinned K split reaches the decode kernel too
+    assert pkg.plan(32, 7168, 2048) == "decode128_k3"      # a pinned K split reaches the decode kernels too
+    pkg.force_config(0, 0)                                 # tile_variant 0 / 1 under this family: narrow / wide strips
+    assert pkg.plan(32, 7168, 2048) == "skinny_k1"
+    assert pkg.plan(32, 1536, 7168) == "skinny_k4"
+    pkg.force_config(1, 2)
+    assert pkg.plan(32, 7168, 2048) == "decode128_k2"
     pkg.force_config(-1, 0)
     pkg.select(pkg.KERNEL_SCALAR)
     assert pkg.plan(8192, 4608, 7168) == "scalar"
@@ -219,6 +226,23 @@ def test_dispatcher_plans(pkg):
     pkg.force_config(1, 4)
     assert pkg.plan(1024, 512, 2048) == "tile256x128_k4"
     pkg.force_config(-1, 0)
+
+
+def test_library_owned_workspace_growth_policy(pkg):
+    """the library-owned workspace at least doubles when it grows: the buffers it retires on the way
+    never add up to more than the live one"""
+    grow = pkg.lib().fp8_block_gemm_workspace_growth
+    assert grow(0, 1000) == 1000 and grow(4096, 100) == 4096 and grow(4096, 4096) == 4096
+    assert grow(4096, 4097) == 8192 and grow(4096, 100000) == 100000
+    have, retired = 0, 0
+    for need in [1 << 10, 3 << 10, 5 << 10, 6 << 10, 7 << 10, 100 << 10, 101 << 10, 1 << 20, (1 << 20) + 1]:
+        new = grow(have, need)
+        assert new >= need
+        if new != have:
+            retired += have
+            have = new
+        assert retired <= have
+    assert grow(2 ** 63 + 5, 2 ** 63 + 6) == 2 ** 64 - 1        # saturates instead of wrapping
 
 
 def test_header_cites_reference_for_every_entry_point(pkg):

@@ -167,6 +167,7 @@ def test_tile_kernel_split_k(pkg, variant, ksplit, m, n, k):
     got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SPLITK, variant=variant, ksplit=ksplit)
     assert name.endswith(f"_k{ksplit}"), name
     _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)   # a partial tile dropped by one split shows here
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 7168, 2048), (16, 96, 512), (32, 576, 7168), (32, 32, 128),
@@ -174,9 +175,10 @@ def test_tile_kernel_split_k(pkg, variant, ksplit, m, n, k):
 def test_skinny_kernel(pkg, m, n, k):
     a, b, sa, sb = oracle.make_inputs(m, n, k, 900 + n)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
-    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=0)   # 0 = the narrow strips
     assert name.startswith("skinny")
     _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
 
 
 @pytest.mark.parametrize("m,n,k,ksplit", [(32, 1536, 7168, 4), (16, 1040, 2048, 2), (32, 576, 7168, 7),
@@ -184,10 +186,88 @@ def test_skinny_kernel(pkg, m, n, k):
 def test_skinny_kernel_with_the_k_range_split_over_workgroups(pkg, m, n, k, ksplit):
     a, b, sa, sb = oracle.make_inputs(m, n, k, 950 + n + ksplit)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
-    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, ksplit=ksplit)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=0, ksplit=ksplit)
     assert name == f"skinny_k{ksplit}", name
     _assert_close(got, ref, name)
     _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+
+
+# wide strips (128 columns), the K splits of a strip added inside the kernel by the last wave to arrive:
+# every K split count the kernel takes, one and two row tiles, a ragged last strip (n % 128 != 0), more
+# strips x splits than CUs (several rounds of workgroups), a single K block per split
+DECODE_STRIP_CASES = [(32, 7168, 2048, 4), (16, 7168, 2048, 4), (32, 7168, 2048, 1), (32, 576, 1024, 3),
+                      (32, 1040, 2048, 16), (16, 96, 512, 2), (32, 128, 128, 1), (32, 4608, 7168, 7),
+                      (16, 1536, 1536, 12), (32, 2048, 384, 3), (32, 16384, 1024, 8), (16, 16, 2048, 6),
+                      (32, 7168, 7168, 14)]
+
+
+@pytest.mark.parametrize("m,n,k,ksplit", DECODE_STRIP_CASES)
+def test_decode_strip_kernel(pkg, m, n, k, ksplit):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1200 + n + k + ksplit, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ksplit)
+    assert name == f"decode128_k{ksplit}", name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    # the sum runs in split order whoever arrives last, and the tickets are zero again after every launch
+    for rep in range(4):
+        again, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ksplit)
+        assert np.array_equal(got, again), f"run {rep}: not reproducible"
+
+
+def test_decode_strip_tickets_survive_a_change_of_shape(pkg):
+    """launches of different strip and split counts back to back share the ticket words"""
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    cases = [(32, 7168, 2048, 4), (16, 1536, 1024, 8), (32, 7168, 2048, 2), (32, 640, 4096, 16), (32, 7168, 2048, 4)]
+    prepared = []
+    for (m, n, k, ks) in cases:
+        a, b, sa, sb = oracle.make_inputs(m, n, k, 1300 + n + ks)
+        prepared.append((oracle.ref_gemm(a, b, sa, sb, m, n, k), _dev(a, b, sa, sb),
+                         torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)))
+    _say(f"[gpu case] decode strips, shapes back to back without a synchronisation: {cases}")
+    pkg.select(pkg.KERNEL_SKINNY)
+    try:
+        for rep in range(3):
+            for (m, n, k, ks), (_, dev, dc) in zip(cases, prepared):
+                pkg.force_config(1, ks)
+                pkg.gemm(dev[0], dev[1], dev[2], dev[3], dc, m, n, k, st)
+    finally:
+        pkg.select(0)
+        pkg.force_config(-1, 0)
+    torch.cuda.synchronize()
+    for (m, n, k, ks), (ref, _, dc) in zip(cases, prepared):
+        _assert_close(dc.cpu().numpy().view(np.uint16), ref, f"decode128_k{ks} {m}x{n}x{k}")
+
+
+def test_decode_strips_in_a_caller_workspace_need_its_zeroed_flag(pkg):
+    """fp8_block_gemm_ex: the in-kernel reduction keeps tickets at the start of the workspace, so a per-call
+    workspace gets it only when the caller vouches for zeroed ticket words; without the flag the call
+    takes a plan that needs none"""
+    import torch
+    m, n, k = 32, 7168, 2048
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1400)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    dev = _dev(a, b, sa, sb)
+    st = torch.cuda.current_stream().cuda_stream
+    need = pkg.workspace_bytes_ex(m, n, k)
+    assert need == pkg.WORKSPACE_HEADER_BYTES + 56 * 4 * 16384
+    ws = torch.full((need,), 0xAB, dtype=torch.uint8, device="cuda")          # garbage, also in the ticket words
+    dc = torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)
+    _say(f"[gpu case] decode in a caller workspace without / with the zeroed flag m={m} n={n} k={k}")
+    pkg.gemm_ex(dev[0], dev[1], dev[2], dev[3], dc, m, n, k, None, ws, need, st)
+    torch.cuda.synchronize()
+    assert not pkg.last_kernel().startswith("decode128_k4"), pkg.last_kernel()
+    _assert_close(dc.cpu().numpy().view(np.uint16), ref, pkg.last_kernel())
+    ws[:pkg.WORKSPACE_HEADER_BYTES] = 0
+    dc.fill_(0x7FC1)
+    opt = pkg.Options(flags=pkg.FLAG_WORKSPACE_ZEROED)
+    for rep in range(3):
+        pkg.gemm_ex(dev[0], dev[1], dev[2], dev[3], dc, m, n, k, opt, ws, need, st)
+    torch.cuda.synchronize()
+    assert pkg.last_kernel() == "decode128_k4", pkg.last_kernel()
+    _assert_close(dc.cpu().numpy().view(np.uint16), ref, "decode128_k4 in a caller workspace")
+    assert int(ws[:pkg.WORKSPACE_HEADER_BYTES].to(torch.int32).sum().item()) == 0, "tickets not back to zero"
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 7168, 7168), (16, 4608, 7168), (32, 1536, 7168), (32, 7168, 4096),
@@ -288,9 +368,10 @@ def test_results_are_bitwise_reproducible(pkg):
         y, _ = _run(pkg, a, b, sa, sb, m, n, k, **kw)
         assert np.array_equal(x, y)
     a, b, sa, sb = oracle.make_inputs(32, 1024, 2048, 32)
-    x, _ = _run(pkg, a, b, sa, sb, 32, 1024, 2048, kernel=4)
-    y, _ = _run(pkg, a, b, sa, sb, 32, 1024, 2048, kernel=4)
-    assert np.array_equal(x, y)
+    for variant in (0, 1):
+        x, _ = _run(pkg, a, b, sa, sb, 32, 1024, 2048, kernel=4, variant=variant)
+        y, _ = _run(pkg, a, b, sa, sb, 32, 1024, 2048, kernel=4, variant=variant)
+        assert np.array_equal(x, y)
 
 
 def test_n576_equals_zero_padded_n640_bit_for_bit(pkg):
@@ -398,7 +479,7 @@ def test_caller_workspace(pkg):
     finally:
         pkg.force_config(-1, 0)
         pkg.select(0)
-    assert need == 8 * m * n * 4
+    assert need == pkg.WORKSPACE_HEADER_BYTES + 8 * m * n * 4
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     pkg.set_workspace(ws, need)
     try:
@@ -489,6 +570,7 @@ def test_grouped_gemm_equals_the_problems_one_by_one(pkg, variant, ms, n, k):
         got = outs[g].cpu().numpy().view(np.uint16)
         ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
         _assert_close(got, ref, f"{name} group {g}")
+        _assert_every_element(got, a, b, sa, sb, m, n, k, f"{name} group {g}")
         single, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=variant, persistent=0)
         assert np.array_equal(got, single), f"group {g}: grouped launch and single launch differ"
 
@@ -518,6 +600,7 @@ def test_grouped_gemm_pads_groups_off_the_16_byte_grid(pkg, ms, n, k):
         if m:
             a, b, sa, sb = host[g]
             _assert_close(got[:m], oracle.ref_gemm(a, b, sa, sb, m, n, k), f"{name} group {g}")
+            _assert_every_element(got[:m], a, b, sa, sb, m, n, k, f"{name} group {g}")
     pkg.release()
 
 
@@ -550,3 +633,4 @@ def test_seeded_sweep_of_shapes_and_plans(pkg):
         got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_AUTO, variant=variant, ksplit=ksplit,
                          persistent=persistent)
         _assert_close(got, ref, f"case {case}: m={m} n={n} k={k} -> {name}")
+        _assert_every_element(got, a, b, sa, sb, m, n, k, f"case {case}: {name}")

@@ -192,3 +192,42 @@ def test_host_launcher_does_not_touch_process_wide_switches(pkg):
         pkg.select(0)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
     assert oracle.compare_bf16(ch, ref, 1e-2, 1e-3)["bad"] == 0
+
+
+def test_library_owned_workspace_growth_keeps_device_memory_bounded(pkg):
+    """K-splitting plans whose need creeps up call by call (a growing batch): the library-owned workspace
+    at least doubles when it grows and frees the buffers it has outgrown once their work is done, so the
+    memory it holds stays within a small multiple of the largest need instead of the sum of all needs"""
+    import torch
+    pkg.set_workspace(None, 0)
+    pkg.release()
+    st = torch.cuda.current_stream().cuda_stream
+    m, k = 1024, 512
+    shapes = [(m, 1024 + 64 * i, k) for i in range(25)]
+    n_max = shapes[-1][1]
+    a, b, sa, sb = oracle.make_inputs(m, n_max, k, 8401)
+    da, dsa = _dev(a, sa)
+    dc = torch.zeros((m, n_max), dtype=torch.int16, device="cuda")
+    pkg.select(pkg.KERNEL_SPLITK)
+    pkg.force_config(2, 4)
+    try:
+        needs = [pkg.workspace_bytes(*s) for s in shapes]
+        assert needs[0] > 16 << 20 and all(x < y for x, y in zip(needs, needs[1:]))
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        _say(f"[gpu case] workspace growth over {len(shapes)} calls, needs {needs[0] >> 20} .. {needs[-1] >> 20} MiB")
+        for (mm, n, kk) in shapes:
+            bn = np.ascontiguousarray(b[:, :n])
+            sbn = np.ascontiguousarray(sb[:, :(n + 127) // 128])
+            db, dsb = _dev(bn, sbn)
+            pkg.gemm(da, db, dsa, dsb, dc[:, :n].contiguous(), mm, n, kk, st)
+            torch.cuda.synchronize()
+            del db, dsb
+        torch.cuda.empty_cache()
+        held = free_before - torch.cuda.mem_get_info()[0]
+        _say(f"[gpu case] held after growth: {held >> 20} MiB; sum of needs {sum(needs) >> 20} MiB")
+        assert held <= 4 * needs[-1] + (64 << 20), (held, needs[-1])
+    finally:
+        pkg.select(0)
+        pkg.force_config(-1, 0)
+    pkg.release()

@@ -1,6 +1,9 @@
 """fp8_block_gemm_noalloc: the entry point whose workspace is a fixed array in the library's device
-image.  Called through the C ABI on plans that use that workspace (a K split, padded copies), twice in
-a row with the second problem smaller, against fp8_block_gemm_stream on the same inputs: bit for bit."""
+image.  Called through the C ABI on plans that use that workspace (a K split, padded copies, the decode
+kernel's tickets and partial patches), twice in a row with the second problem smaller, against
+fp8_block_gemm_stream on the same inputs: bit for bit.  The calls must leave the device's free memory
+and the library-owned workspace untouched, and must work under stream capture, where the stream entry
+point is refused for want of a workspace."""
 import sys
 
 import numpy as np
@@ -16,33 +19,79 @@ def _say(msg):
     sys.stdout.flush()
 
 
-def _both(pkg, m, n, k, seed, expect):
-    import torch
-    a, b, sa, sb = oracle.make_inputs(m, n, k, seed)
-    dev = [torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in (a, b, sa, sb)]
-    c0 = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
-    c1 = torch.full((m, n), -1, dtype=torch.int16, device="cuda")
-    st = torch.cuda.current_stream().cuda_stream
-    _say(f"[gpu case] noalloc m={m} n={n} k={k} plan={pkg.plan(m, n, k)}")
-    pkg.gemm(*dev, c0, m, n, k, st)
-    torch.cuda.synchronize()
-    name0 = pkg.last_kernel()
-    pkg.gemm_noalloc(*dev, c1, m, n, k, st)
-    torch.cuda.synchronize()
-    name1 = pkg.last_kernel()
-    assert name0 == name1 and expect in name1, (name0, name1)
-    assert np.array_equal(c0.cpu().numpy(), c1.cpu().numpy()), name1
-    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
-    assert oracle.compare_bf16(c1.cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0, name1
+CASES = [(2048, 576, 7168, 8501, "_k3"),      # K split: 14 MB of fp32 partials in the fixed array
+         (1024, 512, 7168, 8502, "_k2"),      # a smaller problem right after, same array
+         (250, 300, 512, 8503, "padded_"),    # padded copies
+         (32, 7168, 2048, 8505, "decode128_k4"),   # tickets and partial patches of the decode kernel
+         (16, 1536, 1024, 8506, "decode128_k"),    # fewer strips right after, same tickets
+         (8192, 4608, 256, 8504, "_k1")]      # needs no workspace at all
 
 
 def test_noalloc_entry_point_matches_the_stream_entry_point(pkg):
+    import torch
     pkg.select(0)
     pkg.force_config(-1, 0)
-    _both(pkg, 2048, 576, 7168, 8501, "_k3")       # K split: 14 MB of fp32 partials in the fixed array
-    _both(pkg, 1024, 512, 7168, 8502, "_k2")       # a smaller problem right after, same array
-    _both(pkg, 250, 300, 512, 8503, "padded_")     # padded copies
-    _both(pkg, 8192, 4608, 256, 8504, "_k1")       # needs no workspace at all
+    st = torch.cuda.current_stream().cuda_stream
+    jobs = []
+    for (m, n, k, seed, expect) in CASES:
+        a, b, sa, sb = oracle.make_inputs(m, n, k, seed)
+        dev = [torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in (a, b, sa, sb)]
+        jobs.append(dict(shape=(m, n, k), host=(a, b, sa, sb), dev=dev, expect=expect,
+                         c0=torch.full((m, n), -1, dtype=torch.int16, device="cuda"),
+                         c1=torch.full((m, n), -1, dtype=torch.int16, device="cuda"),
+                         c2=torch.full((m, n), -1, dtype=torch.int16, device="cuda")))
+    # nothing of the library's own on the device: whatever the calls below need has to come from the array
+    pkg.set_workspace(None, 0)
+    pkg.release()
+    # first use in a process loads the library's device image (the array is part of it) and looks at the
+    # device's workgroup placement: done here, before free memory is read
+    wa, wb, wsa, wsb = oracle.make_inputs(32, 256, 256, 8500)
+    wdev = [torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in (wa, wb, wsa, wsb)]
+    wc = torch.zeros((32, 256), dtype=torch.int16, device="cuda")
+    pkg.gemm_noalloc(*wdev, wc, 32, 256, 256, st)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for j in jobs:
+        m, n, k = j["shape"]
+        _say(f"[gpu case] noalloc m={m} n={n} k={k} plan={pkg.plan(m, n, k)}")
+        pkg.gemm_noalloc(*j["dev"], j["c1"], m, n, k, st)
+        j["name1"] = pkg.last_kernel()
+        assert j["expect"] in j["name1"], j["name1"]
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "fp8_block_gemm_noalloc changed the device's free memory"
+
+    # under capture: the stream entry point has no workspace and may not allocate one; noalloc records
+    j = jobs[0]
+    m, n, k = j["shape"]
+    _say(f"[gpu case] noalloc under stream capture m={m} n={n} k={k}")
+    refused = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cst = torch.cuda.current_stream().cuda_stream
+        try:
+            pkg.gemm(*j["dev"], j["c2"], m, n, k, cst)
+        except pkg.Fp8GemmError as exc:
+            refused = exc.code
+        pkg.gemm_noalloc(*j["dev"], j["c2"], m, n, k, cst)
+    assert refused == -4, "the library-owned workspace was there: noalloc did not leave it alone"
+    for rep in range(3):
+        j["c2"].fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(j["c2"].cpu().numpy(), j["c1"].cpu().numpy()), f"replay {rep}"
+    del graph
+
+    # the stream entry point (which allocates) on the same inputs: same plan, same bits
+    for j in jobs:
+        m, n, k = j["shape"]
+        pkg.gemm(*j["dev"], j["c0"], m, n, k, st)
+        torch.cuda.synchronize()
+        assert pkg.last_kernel() == j["name1"], (pkg.last_kernel(), j["name1"])
+        assert np.array_equal(j["c0"].cpu().numpy(), j["c1"].cpu().numpy()), j["name1"]
+        ref = oracle.ref_gemm(*j["host"], m, n, k)
+        assert oracle.compare_bf16(j["c1"].cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0, j["name1"]
+    pkg.release()
 
 
 def test_noalloc_entry_point_refuses_what_does_not_fit(pkg):
