@@ -14,5 +14,5 @@ from .capi import (  # noqa: F401
     quantize_a_1x128, quantize_b_128x128,
     abi_symbols, build, convert_f32_to_e4m3fn, custom_kernel, error_string, force_config, gemm, gemm_ex, gemm_grouped, gemm_noalloc, gemm_scalar, NOALLOC_MAX_BYTES,
     grouped_workspace_bytes, workspace_bytes_ex,
-    last_kernel, lib, lib_path, plan, release, select, set_persistent, set_workspace, workspace_bytes,
+    last_kernel, lib, lib_path, plan, release, select, set_fused_reduction, set_persistent, set_workspace, workspace_bytes,
 )

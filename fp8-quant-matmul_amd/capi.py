@@ -85,6 +85,8 @@ def lib():
     L.fp8_block_gemm_grouped.argtypes = [i, vp, vp, vp, vp, vp, vp, i, i, vp]
     L.fp8_block_gemm_set_persistent.restype = i
     L.fp8_block_gemm_set_persistent.argtypes = [i]
+    L.fp8_block_gemm_set_fused_reduction.restype = i
+    L.fp8_block_gemm_set_fused_reduction.argtypes = [i]
     L.fp8_block_gemm_plan.restype = i
     L.fp8_block_gemm_plan.argtypes = [i, i, i, C.c_char_p, sz]
     L.fp8_block_gemm_last_kernel.restype = C.c_char_p
@@ -200,6 +202,11 @@ def gemm_grouped(a, b, a_scale, b_scale, c, m, n, k, stream=None):
 def set_persistent(mode=-1):
     """-1: persistent tile kernel when tiles outnumber the CUs, 0: never, 1: whenever possible"""
     _check(lib().fp8_block_gemm_set_persistent(mode), "fp8_block_gemm_set_persistent")
+
+
+def set_fused_reduction(mode=-1):
+    """K splits added inside the GEMM kernel: -1 by cost, 0 never (reduction kernel), 1 whenever possible"""
+    _check(lib().fp8_block_gemm_set_fused_reduction(mode), "fp8_block_gemm_set_fused_reduction")
 
 
 def plan(m, n, k):

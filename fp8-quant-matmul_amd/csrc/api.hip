@@ -23,6 +23,7 @@ std::atomic<int> g_selected{FP8GEMM_KERNEL_AUTO};
 std::atomic<int> g_force_variant{-1};
 std::atomic<int> g_force_ksplit{0};
 std::atomic<int> g_persistent{-1};  // -1 = when tiles outnumber the CUs, 0 = never, 1 = whenever possible
+std::atomic<int> g_fused{-1};       // K splits added inside the GEMM kernel: -1 = by cost, 0 = never, 1 = whenever possible
 thread_local const char* t_last_kernel = "none";
 thread_local char t_name_buf[64];
 
@@ -35,8 +36,15 @@ struct Config {
     // plans that add K splits inside the kernel may be chosen: the workspace starts with zeroed ticket
     // words and the device places workgroups on XCDs as those kernels assume (set by run())
     bool fused_ok = true;
+    int fused_mode = -1;  // -1 = by cost, 0 = never, 1 = whenever fused_ok and the plan allows
 };
-Config global_config() { return Config{g_selected.load(), g_force_variant.load(), g_force_ksplit.load(), g_persistent.load()}; }
+Config global_config()
+{
+    Config c{g_selected.load(), g_force_variant.load(), g_force_ksplit.load(), g_persistent.load()};
+    c.fused_mode = g_fused.load();
+    c.fused_ok = c.fused_mode != 0;
+    return c;
+}
 constexpr int MAX_KSPLIT = 16;
 
 // device memory a call may use beyond its operands: fp32 partial sums of plans that split K, padded
@@ -87,6 +95,7 @@ struct Plan {
     bool persistent = false;  // tile families, ksplit == 1: workgroups walk through the tiles
     bool padded = false;      // the plan is for the problem with m and n rounded up to 16 (run_padded)
     bool wide = false;        // decode family: 128-column strips, K splits added inside the kernel (k_decode.hip)
+    bool fused = false;       // tile family, ksplit > 1: the last workgroup of a tile adds the partial tiles (no reduction launch)
 };
 
 // Shapes or addresses the MFMA kernels cannot take (m or n not a multiple of 16, a base not
@@ -168,6 +177,17 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit)
     return cost;
 }
 
+// The in-kernel reduction against the reduction kernel, measured on 11 shapes x 13 split plans (all
+// bit-identical): the last workgroup of a tile reads ksplit partial tiles at the 15-20 bytes per clock
+// one CU takes in, so it pays while that is little -- 64x64 tiles (16 KB per split): 2-30 % faster up
+// to 4 splits, even at 8 -- and loses from 128x128 tiles on (64 KB per split: +2 ... +40 %; 256x192:
+// up to 3 x), where the reduction kernel's 256 CUs read the partials together.
+bool tile_fused_pays(const GemmArgs& g, int variant, int ksplit)
+{
+    (void)g;
+    return variant == TILE_64x64 && ksplit <= 8;
+}
+
 // Shapes whose best measured plan differs from the model's choice: {m, n, k, variant, ksplit}.
 struct TunedShape { int m, n, k, variant, ksplit; };
 constexpr TunedShape kTuned[] = {
@@ -192,6 +212,21 @@ void decide_persistent(const GemmArgs& g, Plan& p, const Config& cfg)
     tile_variant_dims(p.variant, &bm, &bn);
     const long tiles = (long)((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
     p.persistent = mode == 1 || tiles > NUM_CU;
+}
+
+// Whether a tile plan that splits K adds the partial tiles inside the GEMM kernel (the last workgroup of
+// a tile to finish) or leaves them to the reduction kernel.
+void decide_fused(const GemmArgs& g, Plan& p, const Config& cfg)
+{
+    p.fused = false;
+    if (p.ksplit <= 1 || !cfg.fused_ok || cfg.fused_mode == 0)
+        return;
+    int bm, bn;
+    tile_variant_dims(p.variant, &bm, &bn);
+    const long tiles = (long)((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
+    if (tiles > TILE_TICKET_WORDS || (unsigned long long)g.m * g.n * 4ull * p.ksplit > 0x7FFFFFFFull)
+        return;
+    p.fused = cfg.fused_mode == 1 || tile_fused_pays(g, p.variant, p.ksplit);
 }
 
 Plan make_plan(const GemmArgs& g, const Config& cfg)
@@ -294,6 +329,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
                 p.variant = t.variant;
                 p.ksplit = t.ksplit;
                 decide_persistent(g, p, cfg);
+                decide_fused(g, p, cfg);
                 return p;
             }
     double best = 1e300;
@@ -339,6 +375,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
         return p;
     }
     decide_persistent(g, p, cfg);
+    decide_fused(g, p, cfg);
     if (p.variant == TILE_256x192_W4 && !p.persistent)
         p.family = -1;
     return p;
@@ -438,7 +475,7 @@ void plan_name(const Plan& p, char* out, size_t cap)
         snprintf(out, cap, p.wide ? "%sdecode128_k%d" : "%sskinny_k%d", pre, p.ksplit);
     else
         snprintf(out, cap, "%s%s_k%d%s", pre, tile_variant_name(p.variant), p.ksplit,
-                 p.persistent ? "_persistent" : "");
+                 p.persistent ? "_persistent" : (p.fused ? "f" : ""));
 }
 
 // the kernels of a plan on operands they can take; `partial` holds plan_workspace_bytes, `tickets` the
@@ -455,8 +492,8 @@ hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, unsigne
     default: {
         if (p.persistent)
             return launch_tile_persistent(g, p.variant, NUM_CU, stream);
-        hipError_t e = launch_tile(g, p.variant, p.ksplit, partial, stream);
-        if (e == hipSuccess && p.ksplit > 1)
+        hipError_t e = launch_tile(g, p.variant, p.ksplit, partial, p.fused ? tickets : nullptr, stream);
+        if (e == hipSuccess && p.ksplit > 1 && !p.fused)
             e = launch_splitk_reduce(g, p.ksplit, partial, stream);
         return e;
     }
@@ -545,7 +582,8 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
         Config probe = cfg;
         probe.fused_ok = false;
         const Plan with = make_plan(g, cfg), without = make_plan(g, probe);
-        const bool differs = with.family != without.family || with.ksplit != without.ksplit || with.wide != without.wide;
+        const bool differs = with.family != without.family || with.ksplit != without.ksplit ||
+                             with.wide != without.wide || with.fused != without.fused;
         if (differs && !placement_ok(stream))
             cfg.fused_ok = false;
     }
@@ -905,6 +943,14 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
         if (rc != FP8GEMM_OK)
             return rc;
     }
+    return FP8GEMM_OK;
+}
+
+int fp8_block_gemm_set_fused_reduction(int mode)
+{
+    if (mode < -1 || mode > 1)
+        return FP8GEMM_E_KERNEL;
+    g_fused.store(mode);
     return FP8GEMM_OK;
 }
 

@@ -42,8 +42,8 @@ template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
-                 uint16_t* __restrict__ c, float* __restrict__ partial, int M, int lda, int N, int K,
-                 int tiles_m, int tiles_n, int kb_per_split, int group_m)
+                 uint16_t* __restrict__ c, float* __restrict__ partial, unsigned int* __restrict__ tickets,
+                 int M, int lda, int N, int K, int tiles_m, int tiles_n, int kb_per_split, int group_m)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
     // Eight waves copy; WM x WN of them (all eight, or the first four for the smallest tile)
@@ -73,6 +73,8 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     // group_m so that an XCD's co-resident tiles form a block that is about square in bytes).
     const int T = tiles_m * tiles_n;
     const int pid = blockIdx.x;
+    if (pid >= T)  // grid.x is rounded up to a multiple of 8 when the K splits of a tile have to share an XCD
+        return;
     const int xcd = pid & 7, q8 = T >> 3, r8 = T & 7;
     const int logical = xcd * q8 + (xcd < r8 ? xcd : r8) + (pid >> 3);
     const int per_group = group_m * tiles_n;
@@ -348,6 +350,55 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
             }
         }
     }
+
+    // ---- K splits added inside the kernel (tickets != nullptr).  grid.x is a multiple of 8, so the
+    // workgroups of one tile (same blockIdx.x) have linear ids that agree modulo 8 and share an XCD:
+    // the partial tiles meet in that XCD's L2.  Every thread waits for the L2's acknowledgement of its
+    // stores, the workgroup takes a ticket for the tile (workgroup-scope atomic, executed by that L2; it
+    // wraps to zero with the last arrival), and the workgroup that arrived last adds the partial tiles
+    // in split order -- the arithmetic of splitk_reduce_kernel, whoever arrives last -- and stores bf16.
+    if constexpr (SPLIT) {
+        if (tickets != nullptr) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();  // every thread's partial is in L2; nobody reads the staging area any more
+            auto flag = LDS_PTR(unsigned int, smem);
+            if (threadIdx.x == 0)
+                *flag = __builtin_amdgcn_atomic_inc32(tickets + pid, gridDim.y - 1, __ATOMIC_RELAXED, "workgroup");
+            __syncthreads();
+            if (*flag != gridDim.y - 1)
+                return;
+            constexpr int QPR = BN / 4;                    // 16-byte pieces (4 floats) per tile row
+            constexpr int PIECES = BM * QPR / NTHREADS;    // per thread
+            static_assert(BM * QPR % NTHREADS == 0, "whole pieces per thread");
+            const size_t mn = (size_t)M * N;
+            const __amdgpu_buffer_rsrc_t rp = make_rsrc(partial, (uint32_t)(mn * 4u * gridDim.y));
+            v4f sum[PIECES];
+            uint32_t off[PIECES];
+#pragma unroll
+            for (int it = 0; it < PIECES; ++it) {
+                const int idx = it * NTHREADS + (int)threadIdx.x;
+                const int mrow = m0 + idx / QPR, ncol = n0 + (idx % QPR) * 4;
+                off[it] = (mrow < M && ncol < N) ? (uint32_t)(((size_t)mrow * N + ncol) * 4u) : 0x80000000u;
+            }
+            for (int z = 0; z < (int)gridDim.y; ++z) {
+                const uint32_t zoff = (uint32_t)(mn * 4u) * (uint32_t)z;
+#pragma unroll
+                for (int it = 0; it < PIECES; ++it) {  // loads past the L1 (sc1): served by the L2
+                    const v4f p = __builtin_bit_cast(
+                        v4f, __builtin_amdgcn_raw_buffer_load_b128(rp, off[it], zoff, 16));
+                    sum[it] = z == 0 ? p : sum[it] + p;
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < PIECES; ++it)
+                if (off[it] != 0x80000000u) {
+                    uint2 pk;
+                    pk.x = pack_bf16x2(sum[it][0], sum[it][1]);
+                    pk.y = pack_bf16x2(sum[it][2], sum[it][3]);
+                    *reinterpret_cast<uint2*>(c + (off[it] >> 2)) = pk;
+                }
+        }
+    }
 }
 
 // sum of the K-split partials in split order, then bf16
@@ -421,25 +472,30 @@ int choose_group_m(int tiles_m, int tiles_n, int bm, int bn)
 }
 
 template <int BM, int BN, int WM, int WN, int NS>
-hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, hipStream_t s)
+hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, unsigned int* tickets, hipStream_t s)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
     constexpr int LDS_TOTAL = S::LDS_BYTES;
     const int tiles_m = (g.m + BM - 1) / BM, tiles_n = (g.n + BN - 1) / BN;
     const int nkb = g.k / KBLOCK;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
-    dim3 grid(tiles_m * tiles_n, ksplit);
+    const int tiles = tiles_m * tiles_n;
     const int group_m = choose_group_m(tiles_m, tiles_n, BM, BN);
     if (ksplit > 1) {
+        // in-kernel reduction: one ticket per tile, partial tiles addressed with 32-bit offsets
+        if (tickets && (tiles > TILE_TICKET_WORDS || (unsigned long long)g.m * g.n * 4ull * ksplit > 0x7FFFFFFFull))
+            return hipErrorInvalidValue;
+        dim3 grid(tickets ? (tiles + 7) & ~7 : tiles, ksplit);
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
         FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
-                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
+        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale, g.c, partial,
+                           tickets, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
     } else {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
         FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
-        hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale,
-                           g.c, partial, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
+        hipLaunchKernelGGL(kern, dim3(tiles, 1), dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
+                           partial, static_cast<unsigned int*>(nullptr), g.m, leading_dim(g), g.n, g.k, tiles_m,
+                           tiles_n, kb_per_split, group_m);
     }
     return hipGetLastError();
 }
@@ -482,14 +538,15 @@ void tile_variant_dims(int variant, int* bm, int* bn)
     }
 }
 
-hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, hipStream_t s)
+hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, unsigned int* tickets,
+                       hipStream_t s)
 {
     switch (variant) {
-    case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, s);
-    case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, s);
-    case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, s);
-    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, s);
-    case TILE_64x64: return launch_variant<64, 64, 2, 2, 4>(g, ksplit, partial, s);
+    case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, tickets, s);
+    case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, tickets, s);
+    case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, tickets, s);
+    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, tickets, s);
+    case TILE_64x64: return launch_variant<64, 64, 2, 2, 4>(g, ksplit, partial, tickets, s);
     default: return hipErrorInvalidValue;
     }
 }

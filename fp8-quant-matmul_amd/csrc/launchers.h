@@ -46,14 +46,18 @@ inline int leading_dim(const GemmArgs& g) { return g.lda ? g.lda : g.m; }
 hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);
 
 // MFMA tile kernel family.  `variant` picks the workgroup tile; ksplit > 1 writes fp32
-// partial sums to `partial` ([ksplit][m][n]) instead of c and must be followed by
-// launch_splitk_reduce.
+// partial sums to `partial` ([ksplit][m][n]) instead of c.  With tickets == nullptr it must be followed
+// by launch_splitk_reduce; with tickets (TILE_TICKET_WORDS words, zero before the launch and zero again
+// after it) the workgroup of a tile that finishes last adds the partial tiles itself and writes c, with
+// the same arithmetic.  The latter needs xcd_placement_confirmed() and at most TILE_TICKET_WORDS tiles.
 enum TileVariant { TILE_256x192 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_128x192 = 3,
                    TILE_64x64 = 4, TILE_256x192_W4 = 5, TILE_VARIANT_COUNT };
 bool tile_supports(const GemmArgs& g);
 const char* tile_variant_name(int variant);
 void tile_variant_dims(int variant, int* bm, int* bn);
-hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, hipStream_t s);
+constexpr int TILE_TICKET_WORDS = 4096;
+hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, unsigned int* tickets,
+                       hipStream_t s);
 // Persistent form (ksplit = 1 only): `workgroups` (a multiple of 8) workgroups walk through
 // all tiles, the copies of a tile's first K blocks overlap the previous tile's epilogue.
 bool tile_persistent_supports(const GemmArgs& g, int variant);
@@ -85,7 +89,7 @@ hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStrea
 // wide-strip decode kernel (M <= 32): 128-column strips, the K splits of a strip added inside the
 // kernel.  `partial` holds decode_strip_partial_bytes; `tickets` = DECODE_TICKET_WORDS words that are
 // zero before the launch and zero again after it.  ksplit > 1 needs xcd_placement_confirmed().
-constexpr int DECODE_TICKET_WORDS = 4096;
+constexpr int DECODE_TICKET_WORDS = TILE_TICKET_WORDS;
 constexpr int DECODE_MAX_KSPLIT = 16;
 bool decode_strip_supports(const GemmArgs& g);
 size_t decode_strip_partial_bytes(const GemmArgs& g, int ksplit);

@@ -105,6 +105,18 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit);
  * allows.  The reference names such a kernel as future work (/root/reference/README.md:29). */
 int fp8_block_gemm_set_persistent(int mode);
 
+/* Plans that split K ("..._kN") write fp32 partial results; they are added either by a second kernel or
+ * inside the GEMM kernel by the workgroup (decode kernel: the wave) that finishes a tile last ("..._kNf",
+ * "decode128_kN"): the K splits of a tile are placed on one XCD, meet in its L2 and count themselves in
+ * with a ticket, and the last arrival adds the partials in split order, so the result does not depend on
+ * who is last and equals the second kernel's bit for bit.  mode -1 = by cost (default), 0 = never,
+ * 1 = whenever the plan allows.  The first call that could use it on a device looks once at where that
+ * device places workgroups (a probe grid the call waits for; skipped, and the two-kernel form used, while
+ * the stream is being captured and the answer is not known yet).  The reference does not split K
+ * (/root/reference/mn_small.hip:28); its README names filling the CUs for skinny shapes as the open
+ * problem (/root/reference/README.md:161). */
+int fp8_block_gemm_set_fused_reduction(int mode);
+
 /* Grouped GEMM: `groups` independent problems with the same n and k and their own m[g]
  * (ragged M, e.g. the experts of one MoE layer), C[g] = A[g] . B[g]^T with the layouts above.
  * a, b, a_scale, b_scale, c and m are HOST arrays of `groups` entries; the pointers they hold

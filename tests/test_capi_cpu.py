@@ -98,7 +98,7 @@ def test_workspace_contract(pkg):
     assert pkg.workspace_bytes(0, 8, 128) == 0
     assert pkg.workspace_bytes(64, 64, 128) == 0                     # one K block: nothing to split
     assert pkg.workspace_bytes(8192, 4608, 7168) == 0                # plan does not split K
-    assert pkg.plan(1024, 512, 7168) == "tile64x64_k2"
+    assert pkg.plan(1024, 512, 7168) == "tile64x64_k2f"                # f: the K splits are added inside the kernel
     H = pkg.WORKSPACE_HEADER_BYTES                                   # ticket words ahead of every plan's data
     assert pkg.workspace_bytes(1024, 512, 7168) == H + 2 * 1024 * 512 * 4
     assert L.fp8_block_gemm_force_config(2, 8) == 0                  # follows a forced configuration
@@ -206,7 +206,7 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(32, 16384, 7168) == "decode128_k2"     # 128 strips x 2
     assert pkg.plan(32, 128, 128) == "decode128_k1"        # one K block: nothing to split
     assert pkg.workspace_bytes(32, 7168, 2048) == pkg.WORKSPACE_HEADER_BYTES + 56 * 4 * 16384
-    assert pkg.plan(64, 1536, 7168) == "tile64x64_k7"      # a single row of tiles: never fewer than 8 K blocks per split
+    assert pkg.plan(64, 1536, 7168) == "tile64x64_k7f"     # a single row of tiles: never fewer than 8 K blocks per split
     assert pkg.plan(48, 1536, 1536) == "tile64x64_k1"
     pkg.select(pkg.KERNEL_SKINNY)
     pkg.force_config(-1, 3)
@@ -217,6 +217,15 @@ def test_dispatcher_plans(pkg):
     pkg.force_config(1, 2)
     assert pkg.plan(32, 7168, 2048) == "decode128_k2"
     pkg.force_config(-1, 0)
+    pkg.select(pkg.KERNEL_AUTO)
+    pkg.set_fused_reduction(0)                             # reduction kernel instead of the in-kernel reduction
+    try:
+        assert pkg.plan(64, 1536, 7168) == "tile64x64_k7" and pkg.plan(32, 7168, 2048) == "skinny_k1"
+        pkg.set_fused_reduction(1)
+        assert pkg.plan(2048, 576, 7168).endswith("f")
+    finally:
+        pkg.set_fused_reduction(-1)
+    assert not pkg.plan(2048, 576, 7168).endswith("f")     # 128x128 tiles: the reduction kernel is faster
     pkg.select(pkg.KERNEL_SCALAR)
     assert pkg.plan(8192, 4608, 7168) == "scalar"
     pkg.select(pkg.KERNEL_SKINNY)

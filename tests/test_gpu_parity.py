@@ -28,15 +28,16 @@ def _dev(*arrs):
     return [torch.from_numpy(np.ascontiguousarray(x)).cuda() for x in arrs]
 
 
-def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=False, persistent=-1):
+def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=False, persistent=-1, fused=-1):
     import torch
     da, db, dsa, dsb = _dev(a, b, sa, sb)
     dc = torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)  # NaN sentinel
     _say(f"[gpu case] m={m} n={n} k={k} kernel={kernel} variant={variant} ksplit={ksplit} scalar={scalar} "
-         f"persistent={persistent}")
+         f"persistent={persistent} fused={fused}")
     pkg.select(kernel)
     pkg.force_config(variant, ksplit)
     pkg.set_persistent(persistent)
+    pkg.set_fused_reduction(fused)
     try:
         if scalar:
             pkg.gemm_scalar(da, db, dsa, dsb, dc, m, n, k)
@@ -48,6 +49,7 @@ def _run(pkg, a, b, sa, sb, m, n, k, kernel=0, variant=-1, ksplit=0, scalar=Fals
         pkg.select(0)
         pkg.force_config(-1, 0)
         pkg.set_persistent(-1)
+        pkg.set_fused_reduction(-1)
     return dc.cpu().numpy().view(np.uint16), name
 
 
@@ -157,17 +159,27 @@ def test_tile_kernel_one_wave_per_simd(pkg, m, n, k):
     assert np.array_equal(got, again), "run-to-run reproducible"
 
 
+# the last three: more tiles x splits than CUs (several rounds of workgroups meet at the tickets), a tile
+# count that is not a multiple of 8 with ragged edges, many splits of many small tiles
 @pytest.mark.parametrize("variant,ksplit,m,n,k", [(2, 2, 256, 256, 512), (2, 4, 512, 512, 1024),
                                                    (1, 3, 272, 576, 896), (0, 8, 256, 576, 2048),
                                                    (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048), (3, 5, 384, 576, 1280),
-                                                   (4, 3, 208, 336, 768), (4, 2, 64, 64, 256)])
+                                                   (4, 3, 208, 336, 768), (4, 2, 64, 64, 256),
+                                                   (2, 3, 2048, 576, 1536), (4, 4, 1008, 528, 1024), (4, 16, 512, 512, 2048)])
 def test_tile_kernel_split_k(pkg, variant, ksplit, m, n, k):
+    """the K range split over workgroups: partial tiles added by the reduction kernel (fused=0) and by the
+    last workgroup of each tile inside the GEMM kernel (fused=1) -- same sums in the same order"""
     a, b, sa, sb = oracle.make_inputs(m, n, k, m + n + k + ksplit)
     ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
-    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SPLITK, variant=variant, ksplit=ksplit)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SPLITK, variant=variant, ksplit=ksplit, fused=0)
     assert name.endswith(f"_k{ksplit}"), name
     _assert_close(got, ref, name)
     _assert_every_element(got, a, b, sa, sb, m, n, k, name)   # a partial tile dropped by one split shows here
+    for rep in range(3):
+        inside, fname = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SPLITK, variant=variant, ksplit=ksplit,
+                             fused=1)
+        assert fname == name + "f", fname
+        assert np.array_equal(got, inside), f"{fname} run {rep}: differs from the reduction kernel's result"
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 7168, 2048), (16, 96, 512), (32, 576, 7168), (32, 32, 128),
