@@ -56,6 +56,64 @@ inline void row_to_col_major(const std::vector<float>& in, std::vector<float>& o
             out[(size_t)j * rows + i] = in[(size_t)i * cols + j];
 }
 
+// fp32 -> e4m3fn code, round to nearest even, saturating at 448 (host side, for synthetic operands)
+inline uint8_t e4m3fn_from_float(float x)
+{
+    const uint8_t sign = std::signbit(x) ? 0x80 : 0;
+    float ax = std::fabs(x);
+    if (!(ax < 448.f))
+        return sign | 0x7E;
+    if (ax < 0.0009765625f)  // below half the smallest subnormal (2^-10): zero
+        return sign;
+    int e;
+    (void)std::frexp(ax, &e);            // ax = f * 2^e, f in [0.5, 1)
+    int exp = e - 1 < -6 ? -6 : e - 1;   // exponent of the code's binade (subnormals share -6)
+    const float step = std::ldexp(1.f, exp - 3);
+    const float q = std::nearbyint(ax / step);  // default rounding mode: ties to even
+    const float v = q * step;
+    (void)std::frexp(v, &e);
+    exp = e - 1 < -6 ? -6 : e - 1;
+    const int mant = (int)(v / std::ldexp(1.f, exp - 3)) - (v >= 0.015625f ? 8 : 0);
+    const int biased = v >= 0.015625f ? exp + 7 : 0;
+    return sign | (uint8_t)((biased << 3) | mant);
+}
+
+// Operands with the statistics of the benchmark's: standard normal values, A quantised per row and
+// 128-wide K group (scale = amax / 448, /root/reference/quantize.py:43-67), B per 128 x 128 block
+// (quantize.py:16-41), written in the GEMM's layouts (a: m + k*M, b: n + k*N, scales [K/128][.]).
+inline void quantised_normal_operands(std::vector<uint8_t>& a, std::vector<float>& as, std::vector<uint8_t>& b,
+                                      std::vector<float>& bs, size_t M, size_t N, size_t K)
+{
+    std::mt19937 engine(7);
+    std::normal_distribution<float> dist(0.f, 1.f);
+    const size_t nkb = K / 128, sn = (N + 127) / 128;
+    std::vector<float> grp(128 * 128);
+    for (size_t kb = 0; kb < nkb; ++kb)
+        for (size_t m = 0; m < M; ++m) {
+            float amax = 1e-12f;
+            for (int i = 0; i < 128; ++i) {
+                grp[i] = dist(engine);
+                amax = std::fmax(amax, std::fabs(grp[i]));
+            }
+            as[kb * M + m] = amax / 448.f;
+            for (int i = 0; i < 128; ++i)
+                a[m + (kb * 128 + i) * M] = e4m3fn_from_float(grp[i] * (448.f / amax));
+        }
+    for (size_t kb = 0; kb < nkb; ++kb)
+        for (size_t nb = 0; nb < sn; ++nb) {
+            const size_t cols = N - nb * 128 < 128 ? N - nb * 128 : 128;
+            float amax = 1e-12f;
+            for (size_t i = 0; i < 128 * cols; ++i) {
+                grp[i] = dist(engine);
+                amax = std::fmax(amax, std::fabs(grp[i]));
+            }
+            bs[kb * sn + nb] = amax / 448.f;
+            for (size_t kk = 0; kk < 128; ++kk)
+                for (size_t c = 0; c < cols; ++c)
+                    b[nb * 128 + c + (kb * 128 + kk) * N] = e4m3fn_from_float(grp[kk * cols + c] * (448.f / amax));
+        }
+}
+
 // gemmGPU(C, A, B, As, Bs, M, N, K, option) with the reference's argument meaning.
 inline int gemmGPU(std::vector<bf16_bits>& C, const std::vector<float>& A, const std::vector<float>& B,
                    const std::vector<float>& As, const std::vector<float>& Bs, size_t M, size_t N,

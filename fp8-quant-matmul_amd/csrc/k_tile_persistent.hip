@@ -569,8 +569,48 @@ __device__ __forceinline__ void persistent_body(const Problem& one, const GroupT
         // without a wait that would also cover these stores.
         wait_vmcnt<0>();
         __syncthreads();  // every wave has finished reading that slot
-        store_tile([&](int i, int jj, int r) __attribute__((always_inline)) { return acc[i][jj][r]; },
-                   (uint32_t)(slot_fill * S::STAGE), m0, n0, M, c);
+        // (the same steps as store_tile, written out: handed to that lambda through an accessor, the
+        // running sums cost the K loop 9 more registers and the kernel 1-2 % on the headline shape)
+        {
+            const uint32_t staging = (uint32_t)(slot_fill * S::STAGE);
+            int tid = (int)threadIdx.x;
+            asm volatile("" : "+v"(tid));
+            const int lane_e = tid & 63;
+#pragma unroll
+            for (int p = 0; p < BM / PR; ++p) {
+                if (p > 0)
+                    __syncthreads();  // the previous piece has been read out
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    const int prow = wm * TM + 32 * i;
+                    if (prow / PR == p) {
+                        const uint32_t rbase = staging + (uint32_t)((prow - p * PR + (lane_e & 31)) * CROW);
+#pragma unroll
+                        for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                const int col = wn * TN + 32 * jj + 8 * q + 4 * (lane_e >> 5);
+                                v2i pk = {(int)pack_bf16x2(acc[i][jj][4 * q], acc[i][jj][4 * q + 1]),
+                                          (int)pack_bf16x2(acc[i][jj][4 * q + 2], acc[i][jj][4 * q + 3])};
+                                *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
+                            }
+                    }
+                }
+                __syncthreads();
+#pragma unroll
+                for (int it = 0; it < (CHUNKS + NTH - 1) / NTH; ++it) {
+                    const int idx = it * NTH + tid;
+                    const int row = idx / CPR, ch = idx - row * CPR;
+                    const int mrow = m0 + p * PR + row;
+                    const int ncol = n0 + ch * 8;
+                    if (idx < CHUNKS && mrow < M && ncol < N) {
+                        const v2i lo = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16);
+                        const v2i hi = *LDS_PTR(v2i, lds + staging + row * CROW + ch * 16 + 8);
+                        *reinterpret_cast<v4i*>(c + (size_t)mrow * N + ncol) = (v4i){lo.x, lo.y, hi.x, hi.y};
+                    }
+                }
+            }
+        }
         // the next tile's first K block begins with a barrier: the slot is not written again
         // before every lane has read its chunks of the last piece
     }
