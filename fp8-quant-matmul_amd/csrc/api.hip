@@ -164,7 +164,9 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit)
     const int nkb = g.k / 128;
     const int kbs = (nkb + ksplit - 1) / ksplit;
     const double area = (double)bm * bn / 65536.0;
-    const double per_kb = 1.19 * area + 0.267;
+    // (the 256x256 tile measures 3-5 % ahead of 256x192 per flop where both fill their rounds; the fitted
+    // line, extrapolated to its area, would put it 6 % ahead)
+    const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0);
     const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     const long items = (long)tiles * ksplit;
     // two 64x64 workgroups share a CU; counted only for a single row of tiles (M <= 64), where the K
@@ -197,12 +199,17 @@ constexpr TunedShape kTuned[] = {
     {8192, 7168, 2048, TILE_256x192, 1},
 };
 
+// tile shapes that exist in the persistent form only (and run only when asked for by number)
+inline bool persistent_only(int variant) { return variant == TILE_256x192_W4 || variant == TILE_256x256; }
+// ... of which the dispatcher may pick this one by itself
+inline bool persistent_only_auto(int variant) { return variant == TILE_256x256; }
+
 // A persistent launch pays off when a CU gets more than one tile.
 void decide_persistent(const GemmArgs& g, Plan& p, const Config& cfg)
 {
     p.persistent = false;
     const int mode = cfg.persistent;
-    if (p.variant == TILE_256x192_W4) {  // exists in the persistent form only
+    if (persistent_only(p.variant)) {
         p.persistent = p.ksplit == 1 && tile_persistent_supports(g, p.variant);
         return;
     }
@@ -338,12 +345,17 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             continue;
         if (tile_variant_name(v)[4] == '?')
             continue;
-        if (v == TILE_256x192_W4 && fv != v)  // one-wave-per-SIMD form: only when asked for
-            continue;
+        if (persistent_only(v) && fv != v) {
+            // the one-wave-per-SIMD form: only when asked for; the 256x256 tile: when its persistent form can
+            // run (a ring's worth of K blocks) and the persistent kernel is not switched off
+            if (!persistent_only_auto(v) || cfg.persistent == 0 || !tile_persistent_supports(g, v) ||
+                selected == FP8GEMM_KERNEL_SPLITK)
+                continue;
+        }
         if (g.m <= 64 && fv < 0 && selected == FP8GEMM_KERNEL_AUTO && v != TILE_64x64)
             continue;  // a single row of tiles: taller tiles only multiply rows that do not exist
         for (int ks = 1; ks <= MAX_KSPLIT && ks <= nkb; ++ks) {
-            if (v == TILE_256x192_W4 && ks != 1)
+            if (persistent_only(v) && ks != 1)
                 continue;
             if (fk > 0 && ks != (fk < nkb ? fk : nkb))
                 continue;
@@ -376,7 +388,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
     }
     decide_persistent(g, p, cfg);
     decide_fused(g, p, cfg);
-    if (p.variant == TILE_256x192_W4 && !p.persistent)
+    if (persistent_only(p.variant) && !p.persistent)
         p.family = -1;
     return p;
 }

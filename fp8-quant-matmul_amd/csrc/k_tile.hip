@@ -522,6 +522,7 @@ const char* tile_variant_name(int variant)
     case TILE_128x192: return "tile128x192";
     case TILE_64x64: return "tile64x64";
     case TILE_256x192_W4: return "tile256x192w4";
+    case TILE_256x256: return "tile256x256";
     default: return "tile?";
     }
 }
@@ -534,6 +535,7 @@ void tile_variant_dims(int variant, int* bm, int* bn)
     case TILE_256x192_W4: *bm = 256; *bn = 192; break;
     case TILE_128x192: *bm = 128; *bn = 192; break;
     case TILE_64x64: *bm = 64; *bn = 64; break;
+    case TILE_256x256: *bm = 256; *bn = 256; break;
     default: *bm = 128; *bn = 128; break;
     }
 }

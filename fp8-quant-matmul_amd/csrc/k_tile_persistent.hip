@@ -671,6 +671,7 @@ int persistent_stages(int variant)
     case TILE_128x192: return 3;
     case TILE_128x128: return 4;
     case TILE_256x192_W4: return 2;
+    case TILE_256x256: return 2;
     default: return 0;
     }
 }
@@ -693,6 +694,7 @@ hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups
     case TILE_128x192: return launch_persistent_variant<128, 192, 4, 2, 3, 128>(g, workgroups, s);
     case TILE_128x128: return launch_persistent_variant<128, 128, 2, 4, 4, 128>(g, workgroups, s);
     case TILE_256x192_W4: return launch_persistent_variant<256, 192, 2, 2, 2, 64>(g, workgroups, s);
+    case TILE_256x256: return launch_persistent_variant<256, 256, 4, 2, 2, 128>(g, workgroups, s);
     default: return hipErrorInvalidValue;
     }
 }
@@ -701,7 +703,8 @@ hipError_t launch_tile_persistent(const GemmArgs& g, int variant, int workgroups
 bool tile_grouped_supports(const GroupTable& tab, int n, int k, int variant)
 {
     const int stages = persistent_stages(variant);
-    if (stages == 0 || k / KBLOCK < stages - 1 || tab.groups < 1 || tab.groups > GroupTable::MAX_GROUPS)
+    if (stages == 0 || variant == TILE_256x192_W4 ||  // the one-wave-per-SIMD loop is written for a single problem
+        k / KBLOCK < stages - 1 || tab.groups < 1 || tab.groups > GroupTable::MAX_GROUPS)
         return false;
     for (int g = 0; g < tab.groups; ++g) {
         const GemmArgs ga{tab.a[g], tab.b[g], tab.a_scale[g], tab.b_scale[g], tab.c[g], tab.m[g], n, k, tab.lda[g]};
@@ -720,6 +723,7 @@ hipError_t launch_tile_grouped(GroupTable& tab, int n, int k, int variant, int w
     case TILE_256x128: return launch_grouped_variant<256, 128, 4, 2, 3, 128>(tab, n, k, workgroups, s);
     case TILE_128x192: return launch_grouped_variant<128, 192, 4, 2, 3, 128>(tab, n, k, workgroups, s);
     case TILE_128x128: return launch_grouped_variant<128, 128, 2, 4, 4, 128>(tab, n, k, workgroups, s);
+    case TILE_256x256: return launch_grouped_variant<256, 256, 4, 2, 2, 128>(tab, n, k, workgroups, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -51,7 +51,7 @@ hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);
 // after it) the workgroup of a tile that finishes last adds the partial tiles itself and writes c, with
 // the same arithmetic.  The latter needs xcd_placement_confirmed() and at most TILE_TICKET_WORDS tiles.
 enum TileVariant { TILE_256x192 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_128x192 = 3,
-                   TILE_64x64 = 4, TILE_256x192_W4 = 5, TILE_VARIANT_COUNT };
+                   TILE_64x64 = 4, TILE_256x192_W4 = 5, TILE_256x256 = 6, TILE_VARIANT_COUNT };
 bool tile_supports(const GemmArgs& g);
 const char* tile_variant_name(int variant);
 void tile_variant_dims(int variant, int* bm, int* bn);

@@ -92,7 +92,8 @@ int fp8_block_gemm_select(int kernel_id);
 
 /* Pin the MFMA tile kernels to one workgroup tile (0 = 256x192, 1 = 256x128, 2 = 128x128,
  * 3 = 128x192, 4 = 64x64 rows x columns of C, 5 = 256x192 with one wave per SIMD (persistent
- * form only, never chosen automatically); -1 = choose by cost model) and one K-split count
+ * form only, never chosen automatically), 6 = 256x256 (persistent form only, no K split);
+ * -1 = choose by cost model) and one K-split count
  * (0 = choose, at most 16; more returns FP8GEMM_E_KERNEL).  With FP8GEMM_KERNEL_SKINNY selected the
  * first argument picks the decode kernel instead: 0 = 32-column strips, 1 = 128-column strips whose K
  * splits are added inside the kernel, -1 = by cost.  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros

@@ -161,6 +161,36 @@ def test_tile_kernel_one_wave_per_simd(pkg, m, n, k):
 
 # the last three: more tiles x splits than CUs (several rounds of workgroups meet at the tickets), a tile
 # count that is not a multiple of 8 with ragged edges, many splits of many small tiles
+@pytest.mark.parametrize("m,n,k", [(250, 300, 512), (1000, 200, 256), (4000, 3000, 128), (272, 192, 128)])
+def test_tile_kernel_one_wave_per_simd_off_the_grid(pkg, m, n, k):
+    """the generated K loop on padded copies (leading dimension of A and a_scale above m, C written in
+    place), on a last row tile that is partly empty and on a single K block"""
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 7 * m + n + k, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_AUTO, variant=5)
+    assert name.endswith("tile256x192w4_k1_persistent") and name.startswith("padded_") == (m % 16 != 0 or n % 16 != 0), name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    plain, name0 = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_AUTO, variant=0, ksplit=1, persistent=0)
+    assert name0.endswith("tile256x192_k1"), name0
+    assert np.array_equal(got, plain), "both forms fold the same block sums in the same order"
+    pkg.release()
+
+
+@pytest.mark.parametrize("m,n,k", W4_SHAPES + [(256, 256, 128), (4096, 4096, 256), (272, 528, 640)])
+def test_tile_kernel_256x256(pkg, m, n, k):
+    """the 256 x 256 tile (64 x 128 per wave; persistent form only): same block sums, same fold order"""
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 6 * m + n + k, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=6)
+    assert name == "tile256x256_k1_persistent", name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    plain, name0 = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_LARGE, variant=0, persistent=0)
+    assert name0 == "tile256x192_k1", name0
+    assert np.array_equal(got, plain), "both tiles fold the same block sums in the same order"
+
+
 @pytest.mark.parametrize("variant,ksplit,m,n,k", [(2, 2, 256, 256, 512), (2, 4, 512, 512, 1024),
                                                    (1, 3, 272, 576, 896), (0, 8, 256, 576, 2048),
                                                    (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048), (3, 5, 384, 576, 1280),
@@ -570,6 +600,7 @@ def _grouped_case(pkg, ms, n, k, variant, seed):
                                             (0, [4096, 272, 2048, 1024, 16], 1536, 512),
                                             (1, [512] * 9 + [48, 2064], 1024, 384),
                                             (3, [144] * 40, 384, 640),
+                                            (6, [2048, 272, 16, 1024, 4096], 1280, 512),
                                             (2, [128], 128, 384)])
 def test_grouped_gemm_equals_the_problems_one_by_one(pkg, variant, ms, n, k):
     host, dev, outs, name = _grouped_case(pkg, ms, n, k, variant, 7000 + n + k)
@@ -614,6 +645,16 @@ def test_grouped_gemm_pads_groups_off_the_16_byte_grid(pkg, ms, n, k):
             _assert_close(got[:m], oracle.ref_gemm(a, b, sa, sb, m, n, k), f"{name} group {g}")
             _assert_every_element(got[:m], a, b, sa, sb, m, n, k, f"{name} group {g}")
     pkg.release()
+
+
+def test_grouped_gemm_with_a_tile_shape_that_has_no_grouped_form(pkg):
+    """tile variant 5 pinned (its K loop is written for a single problem): the groups run one by one"""
+    ms, n, k = [256, 528, 48], 384, 256
+    host, dev, outs, name = _grouped_case(pkg, ms, n, k, 5, 8250)
+    assert name == "tile256x192w4_k1_persistent", name
+    for g, m in enumerate(ms):
+        a, b, sa, sb = host[g]
+        _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
 
 
 def test_grouped_gemm_takes_more_groups_than_one_launch_holds(pkg):
