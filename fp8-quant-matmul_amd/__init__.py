@@ -12,7 +12,7 @@ from .capi import (  # noqa: F401
     KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY,
     DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH, FLAG_WORKSPACE_ZEROED, WORKSPACE_HEADER_BYTES,
     quantize_a_1x128, quantize_b_128x128,
-    abi_symbols, build, convert_f32_to_e4m3fn, custom_kernel, error_string, force_config, gemm, gemm_ex, gemm_grouped, gemm_noalloc, gemm_scalar, NOALLOC_MAX_BYTES,
+    abi_symbols, build, convert_f32_to_e4m3fn, custom_kernel, error_string, force_config, gemm, gemm_ex, gemm_grouped, gemm_grouped_ex, gemm_noalloc, gemm_scalar, NOALLOC_MAX_BYTES,
     grouped_workspace_bytes, workspace_bytes_ex,
     last_kernel, lib, lib_path, plan, release, select, set_fused_reduction, set_persistent, set_workspace, workspace_bytes,
 )

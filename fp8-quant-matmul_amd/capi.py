@@ -15,7 +15,7 @@ _LIB = None
 KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5)
 DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH = 0, 1, 2
 FLAG_WORKSPACE_ZEROED = 1
-WORKSPACE_HEADER_BYTES = 16384
+WORKSPACE_HEADER_BYTES = 16384 + (8 << 20)
 
 
 class Options(C.Structure):
@@ -73,6 +73,10 @@ def lib():
     L.fp8_block_gemm_workspace_bytes_ex.argtypes = [i, i, i, C.POINTER(Options), i]
     L.fp8_block_gemm_grouped_workspace_bytes.restype = sz
     L.fp8_block_gemm_grouped_workspace_bytes.argtypes = [i, C.POINTER(C.c_int), i, i]
+    L.fp8_block_gemm_grouped_workspace_bytes_ex.restype = sz
+    L.fp8_block_gemm_grouped_workspace_bytes_ex.argtypes = [i, C.POINTER(C.c_int), i, i, C.POINTER(Options)]
+    L.fp8_block_gemm_grouped_ex.restype = i
+    L.fp8_block_gemm_grouped_ex.argtypes = [i, vp, vp, vp, vp, vp, vp, i, i, C.POINTER(Options), vp, sz, vp]
     L.fp8_block_gemm_noalloc.restype = i
     L.fp8_block_gemm_noalloc.argtypes = [vp, vp, fp, fp, vp, i, i, i, vp]
     L.fp8_block_gemm_scalar.restype = i
@@ -168,9 +172,14 @@ def workspace_bytes_ex(m, n, k, options=None, any_alignment=False):
     return int(lib().fp8_block_gemm_workspace_bytes_ex(m, n, k, opt, 1 if any_alignment else 0))
 
 
-def grouped_workspace_bytes(m, n, k):
+def grouped_workspace_bytes(m, n, k, options=None, per_call=False):
+    """Workspace bound of gemm_grouped (process-wide switches), or of gemm_grouped_ex under `options`
+    when options is given or per_call is set."""
     ms = (C.c_int * len(m))(*[int(v) for v in m])
-    return int(lib().fp8_block_gemm_grouped_workspace_bytes(len(m), ms, n, k))
+    if options is None and not per_call:
+        return int(lib().fp8_block_gemm_grouped_workspace_bytes(len(m), ms, n, k))
+    opt = C.byref(options) if options is not None else None
+    return int(lib().fp8_block_gemm_grouped_workspace_bytes_ex(len(m), ms, n, k, opt))
 
 
 def gemm_scalar(a, b, a_scale, b_scale, c, m, n, k, stream=None):
@@ -197,6 +206,19 @@ def gemm_grouped(a, b, a_scale, b_scale, c, m, n, k, stream=None):
     ms = (C.c_int * groups)(*[int(v) for v in m])
     _check(lib().fp8_block_gemm_grouped(groups, ptrs(a), ptrs(b), ptrs(a_scale), ptrs(b_scale), ptrs(c),
                                         ms, n, k, stream), "fp8_block_gemm_grouped")
+
+
+def gemm_grouped_ex(a, b, a_scale, b_scale, c, m, n, k, options=None, workspace=None, workspace_bytes=0, stream=None):
+    """Per-call form of gemm_grouped: `options` and `workspace` as for gemm_ex; allocates nothing and
+    reads no process-wide switch."""
+    groups = len(m)
+    if not (len(a) == len(b) == len(a_scale) == len(b_scale) == len(c) == groups):
+        raise ValueError("one entry per group in every list")
+    ptrs = lambda xs: (C.c_void_p * groups)(*[_ptr(x) for x in xs])
+    ms = (C.c_int * groups)(*[int(v) for v in m])
+    opt = C.byref(options) if options is not None else None
+    _check(lib().fp8_block_gemm_grouped_ex(groups, ptrs(a), ptrs(b), ptrs(a_scale), ptrs(b_scale), ptrs(c), ms, n, k,
+                                           opt, _ptr(workspace), workspace_bytes, stream), "fp8_block_gemm_grouped_ex")
 
 
 def set_persistent(mode=-1):

@@ -49,16 +49,20 @@ constexpr int MAX_KSPLIT = 16;
 
 // device memory a call may use beyond its operands: fp32 partial sums of plans that split K, padded
 // copies of operands off the 16-byte grid
-// The first WS_HEADER bytes hold the arrival tickets of the kernels that add their K splits
-// themselves (zero before the first call and after every call); plans keep their data behind it.
+// The first WS_HEADER bytes belong to the kernels that add their K splits themselves and are zero before
+// the first call and after every call: the arrival tickets of the tile kernels, then the mailbox through
+// which the decode kernel's splits hand over their partial patches.  Plans keep their data behind it.
 struct Workspace {
     float* ptr;
     size_t bytes;
     bool zeroed;  // the header was zero-filled when the buffer was taken on and only this library wrote to it since
 };
-constexpr size_t WS_HEADER = (size_t)DECODE_TICKET_WORDS * sizeof(unsigned int);
+constexpr size_t WS_TICKET_BYTES = (size_t)TILE_TICKET_WORDS * sizeof(unsigned int);
+constexpr size_t WS_HEADER = WS_TICKET_BYTES + DECODE_MAILBOX_BYTES;
+static_assert(WS_HEADER == FP8GEMM_WORKSPACE_HEADER_BYTES, "the header size is part of the ABI");
 inline float* ws_data(const Workspace& w) { return w.ptr ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(w.ptr) + WS_HEADER) : nullptr; }
 inline unsigned int* ws_tickets(const Workspace& w) { return reinterpret_cast<unsigned int*>(w.ptr); }
+inline float* ws_mailbox(const Workspace& w) { return w.ptr ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(w.ptr) + WS_TICKET_BYTES) : nullptr; }
 
 std::mutex g_ws_mutex;
 float* g_ws_own = nullptr;       // library-owned workspace
@@ -277,7 +281,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             // the unsplit form exists
             const int hi = cfg.fused_ok ? (nkb < MAX_KSPLIT ? nkb : MAX_KSPLIT) : 1;
             for (int ks = 1; ks <= hi; ++ks) {
-                if (!valid_split(ks) || (forced_ks && ks != forced_ks))
+                if (!valid_split(ks) || (forced_ks && ks != forced_ks) || !decode_strip_can_split(g, ks))
                     continue;
                 const double cst = decode_strip_cost(g, ks);
                 if (cst < wide_us) {
@@ -290,6 +294,11 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
         // ahead of the narrow ones and of every tile plan on all 40 shapes measured (M = 16, 32; N = 1536 ...
         // 16384; K = 1536 ... 7168: 6.0-27 us against 7.3-60 us), although the narrow kernel is 1-2 us faster
         // on short K when B happens to sit in the Infinity Cache.  They need the in-kernel reduction.
+        // With more than 32 rows the 64x64 tile plans that add their K splits in the kernel are ahead of the wide
+        // strips on 22 of 24 shapes (M = 48, 64; same N and K; from HBM 6.2-15 us against 7.5-16 us): the
+        // four-row-tile form is there for grouped launches and runs single problems only when asked for by name.
+        if (!by_name && g.m > 32)
+            wide_us = 1e300;
         if (!by_name && cfg.force_variant < 0 && cfg.force_ksplit <= 0 && wide_us < 1e300 && cfg.fused_ok)
             return wide;
         if (!by_name && !cfg.fused_ok)
@@ -469,14 +478,14 @@ int acquire_workspace(size_t bytes, hipStream_t stream, Workspace* out)
 // bytes of partial sums a plan keeps behind the workspace header
 size_t plan_workspace_bytes(const GemmArgs& g, const Plan& p)
 {
-    if (p.ksplit <= 1)
+    if (p.ksplit <= 1 || (p.family == FP8GEMM_KERNEL_SKINNY && p.wide))  // the decode kernel's splits meet in the header
         return 0;
-    if (p.family == FP8GEMM_KERNEL_SKINNY && p.wide)
-        return decode_strip_partial_bytes(g, p.ksplit);
     return (size_t)p.ksplit * g.m * g.n * sizeof(float);
 }
+// whether a plan uses the header although it keeps nothing behind it
+inline bool plan_uses_header(const Plan& p) { return p.family == FP8GEMM_KERNEL_SKINNY && p.wide && p.ksplit > 1; }
 // a workspace that holds `data` bytes of a plan: nothing, or the header and the data
-inline size_t with_header(size_t data) { return data ? data + WS_HEADER : 0; }
+inline size_t with_header(size_t data, bool header_alone = false) { return data || header_alone ? data + WS_HEADER : 0; }
 
 void plan_name(const Plan& p, char* out, size_t cap)
 {
@@ -490,16 +499,17 @@ void plan_name(const Plan& p, char* out, size_t cap)
                  p.persistent ? "_persistent" : (p.fused ? "f" : ""));
 }
 
-// the kernels of a plan on operands they can take; `partial` holds plan_workspace_bytes, `tickets` the
-// zeroed words of the workspace header (plans that add their K splits inside the kernel)
-hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, unsigned int* tickets, hipStream_t stream)
+// the kernels of a plan on operands they can take; `partial` holds plan_workspace_bytes, `w` is the
+// workspace whose zeroed header the plans use that add their K splits inside the kernel
+hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, const Workspace& w, hipStream_t stream)
 {
+    unsigned int* const tickets = ws_tickets(w);
     switch (p.family) {
     case FP8GEMM_KERNEL_SCALAR:
         return launch_scalar(g, stream);
     case FP8GEMM_KERNEL_SKINNY:
         if (p.wide)
-            return launch_decode_strips(g, p.ksplit, partial, tickets, stream);
+            return launch_decode_strips(g, p.ksplit, ws_mailbox(w), stream);
         return launch_skinny(g, p.ksplit, partial, stream);
     default: {
         if (p.persistent)
@@ -520,7 +530,7 @@ size_t padded_bytes(const GemmArgs& g, const Plan& p)
     gp.m = (g.m + 15) & ~15;
     gp.n = (g.n + 15) & ~15;
     const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK;
-    return with_header(pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows).total);
+    return with_header(pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows).total, plan_uses_header(p));
 }
 
 int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t stream)
@@ -556,7 +566,7 @@ int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t
     if (L.c)
         gp.c = reinterpret_cast<uint16_t*>(base + L.off_c);
     if (e == hipSuccess)
-        e = launch_plan(gp, p, reinterpret_cast<float*>(base + L.off_partial), ws_tickets(w), stream);
+        e = launch_plan(gp, p, reinterpret_cast<float*>(base + L.off_partial), w, stream);
     if (e == hipSuccess && L.c)
         e = launch_crop_bf16(gp.c, g.c, g.m, g.n, gp.n, stream);
     return (int)e;
@@ -602,7 +612,7 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
     const Plan p = make_plan(g, cfg);
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
-    const size_t need = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p));
+    const size_t need = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p), plan_uses_header(p));
     Workspace w{nullptr, 0, false};
     if (need) {
         if (explicit_ws) {
@@ -616,7 +626,7 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
                 return rc;
         }
     }
-    const int rc = p.padded ? run_padded(g, p, w, stream) : (int)launch_plan(g, p, ws_data(w), ws_tickets(w), stream);
+    const int rc = p.padded ? run_padded(g, p, w, stream) : (int)launch_plan(g, p, ws_data(w), w, stream);
     if (rc == FP8GEMM_OK) {
         plan_name(p, t_name_buf, sizeof(t_name_buf));
         t_last_kernel = t_name_buf;
@@ -655,8 +665,8 @@ int scratch_for_current_device(void** out)
 }
 
 // tile shape for a grouped launch: what the cost model picks for the stacked problem, among the
-// shapes that have a persistent form, without a K split; -1 when none can take the table
-int grouped_variant(const GroupTable& tab, int n, int k)
+// shapes that have a grouped form, without a K split; -1 when none can take the table
+int grouped_variant(const GroupTable& tab, int n, int k, const Config& cfg)
 {
     long long m_total = 0;
     for (int g = 0; g < tab.groups; ++g)
@@ -665,7 +675,7 @@ int grouped_variant(const GroupTable& tab, int n, int k)
         return -1;
     int best_v = -1;
     double best = 1e300;
-    const int fv = g_force_variant.load();
+    const int fv = cfg.force_variant;
     const GemmArgs stacked{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], (int)m_total, n, k};
     for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
         if ((fv >= 0 && v != fv) || !tile_grouped_supports(tab, n, k, v))
@@ -679,77 +689,139 @@ int grouped_variant(const GroupTable& tab, int n, int k)
     return best_v;
 }
 
-// Grouped launch for problems off the 16-byte grid: A and a_scale of every group (B and C too
-// when n or one of their addresses is off the grid) go through padded copies in the workspace,
-// one batched copy launch per kind around one grouped GEMM.  Returns GROUPED_NOT_APPLICABLE when it cannot run
-// (the caller then takes the groups one by one).
+// the workspace of a call: the caller's per-call one, else the process-wide one
+int workspace_for(size_t need, hipStream_t stream, const Workspace* explicit_ws, Workspace* out)
+{
+    *out = Workspace{nullptr, 0, false};
+    if (!need)
+        return FP8GEMM_OK;
+    if (explicit_ws) {
+        if (!explicit_ws->ptr || explicit_ws->bytes < need || (reinterpret_cast<uintptr_t>(explicit_ws->ptr) % 256) != 0)
+            return FP8GEMM_E_WORKSPACE;
+        *out = *explicit_ws;
+        return FP8GEMM_OK;
+    }
+    return acquire_workspace(need, stream, out);
+}
+
+// One grouped launch for the problems of `tab` (same n and k): the decode kernel when every group has at
+// most 64 rows (decode = true), else the persistent tile kernel.  Groups off the 16-byte grid (m or n not a
+// multiple of 16, an operand off a 16-byte boundary) run on zero-padded copies in the workspace made by one
+// batched copy launch per operand kind.  Returns GROUPED_NOT_APPLICABLE when it cannot run (the caller
+// then takes the groups one by one).
 constexpr int GROUPED_NOT_APPLICABLE = -1000;
-int run_grouped_padded(const GroupTable& tab, int n, int k, hipStream_t s)
+int run_grouped_table(const GroupTable& tab, int n, int k, bool decode, hipStream_t s, const Config& cfg,
+                      const Workspace* explicit_ws)
 {
     const long long lim = 0x7FFFFFFFll;
     const int n16 = (n + 15) & ~15;
     const size_t nkb = (size_t)k / 128;
-    bool pad_b = n16 != n, pad_c = n16 != n;
+    bool pad_a = false, pad_b = n16 != n, pad_c = n16 != n;
     for (int g = 0; g < tab.groups; ++g) {
+        pad_a = pad_a || tab.m[g] % 16 != 0 || misaligned16(tab.a[g]) || misaligned16(tab.a_scale[g]);
         pad_b = pad_b || misaligned16(tab.b[g]);
         pad_c = pad_c || misaligned16(tab.c[g]);
     }
+    const bool padded = pad_a || pad_b || pad_c;
     size_t off_a[GroupTable::MAX_GROUPS], off_as[GroupTable::MAX_GROUPS], off_b[GroupTable::MAX_GROUPS],
         off_c[GroupTable::MAX_GROUPS];
     size_t off = 0;
-    for (int g = 0; g < tab.groups; ++g) {
-        const long long m16 = (tab.m[g] + 15) & ~15;
-        if (m16 * k > lim || (long long)n16 * k > lim || m16 * n16 > lim)
+    if (padded)
+        for (int g = 0; g < tab.groups; ++g) {
+            const long long m16 = (tab.m[g] + 15) & ~15;
+            if (m16 * k > lim || (long long)n16 * k > lim || m16 * n16 > lim)
+                return GROUPED_NOT_APPLICABLE;
+            off_a[g] = off;
+            off += round256((size_t)k * m16);
+            off_as[g] = off;
+            off += round256(nkb * m16 * sizeof(float));
+            off_b[g] = off;
+            off += pad_b ? round256((size_t)k * n16) : 0;
+            off_c[g] = off;
+            off += pad_c ? round256((size_t)m16 * n16 * 2) : 0;
+        }
+    // the problems as the GEMM kernel sees them (addresses in the workspace are filled in below): c in place
+    // keeps its m rows, a and a_scale have m16 per k-row
+    GroupTable pt = tab;
+    if (padded)
+        for (int g = 0; g < tab.groups; ++g) {
+            const int m16 = (tab.m[g] + 15) & ~15;
+            pt.m[g] = pad_c ? m16 : tab.m[g];
+            pt.lda[g] = m16;
+        }
+    // decode kernel: K split by cost (it needs the zeroed mailbox and the XCD placement); tile kernel: none
+    int ksplit = 1;
+    int variant = -1;
+    if (decode) {
+        // placeholder addresses that pass the alignment checks while the real ones are not known yet
+        GroupTable probe = pt;
+        if (padded)
+            for (int g = 0; g < tab.groups; ++g) {
+                probe.a[g] = reinterpret_cast<const uint8_t*>(uintptr_t(4096));
+                probe.a_scale[g] = reinterpret_cast<const float*>(uintptr_t(4096));
+                if (pad_b)
+                    probe.b[g] = reinterpret_cast<const uint8_t*>(uintptr_t(4096));
+                if (pad_c)
+                    probe.c[g] = reinterpret_cast<uint16_t*>(uintptr_t(4096));
+            }
+        if (!decode_grouped_supports(probe, n16, k))
             return GROUPED_NOT_APPLICABLE;
-        off_a[g] = off;
-        off += round256((size_t)k * m16);
-        off_as[g] = off;
-        off += round256(nkb * m16 * sizeof(float));
-        off_b[g] = off;
-        off += pad_b ? round256((size_t)k * n16) : 0;
-        off_c[g] = off;
-        off += pad_c ? round256((size_t)m16 * n16 * 2) : 0;
+        bool fused_ok = cfg.fused_ok && (!explicit_ws || explicit_ws->zeroed);
+        if (fused_ok && decode_grouped_ksplit(pt, n16, k, true) > 1)
+            fused_ok = placement_ok(s);
+        ksplit = cfg.force_ksplit > 0 && fused_ok ? cfg.force_ksplit : decode_grouped_ksplit(pt, n16, k, fused_ok);
+        const int nkb_i = k / 128;
+        while (ksplit > 1 && (ksplit > nkb_i || (ksplit - 1) * ((nkb_i + ksplit - 1) / ksplit) >= nkb_i))
+            --ksplit;
+        if (decode_grouped_mailbox_bytes(pt, n16, ksplit) > DECODE_MAILBOX_BYTES)
+            ksplit = 1;
     }
-    Workspace w{nullptr, 0, false};
-    const int wrc = acquire_workspace(with_header(off), s, &w);
+    Workspace w;
+    const int wrc = workspace_for(with_header(off, ksplit > 1), s, explicit_ws, &w);
     if (wrc == FP8GEMM_E_WORKSPACE)
-        return GROUPED_NOT_APPLICABLE;  // a caller-supplied workspace sized for single problems: one by one
+        return GROUPED_NOT_APPLICABLE;  // a workspace sized for single problems: one by one
     if (wrc != FP8GEMM_OK)
         return wrc;
     uint8_t* base = reinterpret_cast<uint8_t*>(ws_data(w));
-    GroupTable pt;
     RepackTable ta, tas, tb, tc;
-    pt.groups = ta.groups = tas.groups = tb.groups = tc.groups = tab.groups;
-    for (int g = 0; g < tab.groups; ++g) {
-        const int m = tab.m[g], m16 = (m + 15) & ~15;
-        pt.a[g] = base + off_a[g];
-        pt.a_scale[g] = reinterpret_cast<const float*>(base + off_as[g]);
-        pt.b[g] = pad_b ? base + off_b[g] : tab.b[g];
-        pt.b_scale[g] = tab.b_scale[g];
-        // c in place keeps its m rows; a and a_scale have m16 per k-row either way
-        pt.c[g] = pad_c ? reinterpret_cast<uint16_t*>(base + off_c[g]) : tab.c[g];
-        pt.m[g] = pad_c ? m16 : m;
-        pt.lda[g] = m16;
-        ta.src[g] = tab.a[g], ta.dst[g] = base + off_a[g], ta.rows[g] = k, ta.ld_src[g] = m, ta.ld_dst[g] = m16;
-        tas.src[g] = tab.a_scale[g], tas.dst[g] = base + off_as[g], tas.rows[g] = (int)nkb, tas.ld_src[g] = m,
-        tas.ld_dst[g] = m16;
-        tb.src[g] = tab.b[g], tb.dst[g] = base + off_b[g], tb.rows[g] = k, tb.ld_src[g] = n, tb.ld_dst[g] = n16;
-        tc.src[g] = base + off_c[g], tc.dst[g] = tab.c[g], tc.rows[g] = m, tc.ld_src[g] = n16, tc.ld_dst[g] = n;
+    ta.groups = tas.groups = tb.groups = tc.groups = tab.groups;
+    if (padded)
+        for (int g = 0; g < tab.groups; ++g) {
+            const int m = tab.m[g], m16 = (m + 15) & ~15;
+            pt.a[g] = base + off_a[g];
+            pt.a_scale[g] = reinterpret_cast<const float*>(base + off_as[g]);
+            pt.b[g] = pad_b ? base + off_b[g] : tab.b[g];
+            pt.c[g] = pad_c ? reinterpret_cast<uint16_t*>(base + off_c[g]) : tab.c[g];
+            ta.src[g] = tab.a[g], ta.dst[g] = base + off_a[g], ta.rows[g] = k, ta.ld_src[g] = m, ta.ld_dst[g] = m16;
+            tas.src[g] = tab.a_scale[g], tas.dst[g] = base + off_as[g], tas.rows[g] = (int)nkb, tas.ld_src[g] = m,
+            tas.ld_dst[g] = m16;
+            tb.src[g] = tab.b[g], tb.dst[g] = base + off_b[g], tb.rows[g] = k, tb.ld_src[g] = n, tb.ld_dst[g] = n16;
+            tc.src[g] = base + off_c[g], tc.dst[g] = tab.c[g], tc.rows[g] = m, tc.ld_src[g] = n16, tc.ld_dst[g] = n;
+        }
+    if (!decode) {
+        variant = grouped_variant(pt, n16, k, cfg);
+        if (variant < 0)
+            return GROUPED_NOT_APPLICABLE;
     }
-    const int v = grouped_variant(pt, n16, k);
-    if (v < 0)
-        return GROUPED_NOT_APPLICABLE;
-    hipError_t e = launch_pad_bytes_batched(ta, s);
+    hipError_t e = hipSuccess;
+    if (padded) {
+        e = launch_pad_bytes_batched(ta, s);
+        if (e == hipSuccess)
+            e = launch_pad_floats_batched(tas, s);
+        if (e == hipSuccess && pad_b)
+            e = launch_pad_bytes_batched(tb, s);
+    }
     if (e == hipSuccess)
-        e = launch_pad_floats_batched(tas, s);
-    if (e == hipSuccess && pad_b)
-        e = launch_pad_bytes_batched(tb, s);
-    if (e == hipSuccess)
-        e = launch_tile_grouped(pt, n16, k, v, NUM_CU, s);
+        e = decode ? launch_decode_grouped(pt, n16, k, ksplit, ws_mailbox(w), s)
+                   : launch_tile_grouped(pt, n16, k, variant, NUM_CU, s);
     if (e == hipSuccess && pad_c)
         e = launch_crop_bf16_batched(tc, s);
     if (e == hipSuccess) {
-        snprintf(t_name_buf, sizeof(t_name_buf), "padded_%s_k1_grouped%d", tile_variant_name(v), tab.groups);
+        if (decode)
+            snprintf(t_name_buf, sizeof(t_name_buf), "%sdecode128_k%d_grouped%d", padded ? "padded_" : "", ksplit, tab.groups);
+        else
+            snprintf(t_name_buf, sizeof(t_name_buf), "%s%s_k1_grouped%d", padded ? "padded_" : "", tile_variant_name(variant),
+                     tab.groups);
         t_last_kernel = t_name_buf;
     }
     return (int)e;
@@ -784,7 +856,7 @@ size_t workspace_bytes_for(int m, int n, int k, const Config& cfg, bool any_alig
     size_t need = 0;
     if (p.family >= 0)
         need = with_header(p.padded ? pad_layout(g, plan_workspace_bytes(gp, p), true, false).total
-                                    : plan_workspace_bytes(g, p));
+                                    : plan_workspace_bytes(g, p), plan_uses_header(p));
     if (any_alignment && !(p.family >= 0 && p.padded)) {
         // the same shape with an operand off a 16-byte boundary: the plan of the padded shape on copies
         const long long lim = 0x7FFFFFFFll;
@@ -792,7 +864,7 @@ size_t workspace_bytes_for(int m, int n, int k, const Config& cfg, bool any_alig
             cfg.selected != FP8GEMM_KERNEL_SCALAR) {
             const Plan pp = make_plan(gp, cfg);
             if (pp.family >= 0 && pp.family != FP8GEMM_KERNEL_SCALAR) {
-                const size_t all = with_header(pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total);
+                const size_t all = with_header(pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total, plan_uses_header(pp));
                 need = all > need ? all : need;
             }
         }
@@ -854,7 +926,7 @@ int fp8_block_gemm_noalloc(const void* a, const void* b, const float* a_scale, c
         const Plan p = make_plan(g, probe);
         if (p.family < 0)
             return FP8GEMM_E_KERNEL;
-        const size_t bytes = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p));
+        const size_t bytes = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p), plan_uses_header(p));
         need = bytes > need ? bytes : need;
     }
     if (need > (size_t)FP8GEMM_NOALLOC_MAX_BYTES)
@@ -863,7 +935,7 @@ int fp8_block_gemm_noalloc(const void* a, const void* b, const float* a_scale, c
     const int rc = scratch_for_current_device(&ptr);
     if (rc != FP8GEMM_OK)
         return rc;
-    // the array starts out zero and every kernel that uses the ticket words leaves them zero
+    // the array starts out zero and every kernel that uses the header leaves it zero
     const Workspace w{static_cast<float*>(ptr), (size_t)FP8GEMM_NOALLOC_MAX_BYTES, true};
     return run(a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), cfg, &w);
 }
@@ -892,9 +964,11 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit)
     return FP8GEMM_OK;
 }
 
-int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* b,
-                           const float* const* a_scale, const float* const* b_scale,
-                           void* const* c, const int* m, int n, int k, void* stream)
+// Grouped GEMM behind both entry points.  explicit_ws = the caller's per-call workspace, nullptr = the
+// process-wide one.
+static int run_grouped(int groups, const void* const* a, const void* const* b, const float* const* a_scale,
+                       const float* const* b_scale, void* const* c, const int* m, int n, int k, hipStream_t s,
+                       const Config& cfg, const Workspace* explicit_ws)
 {
     if (groups < 0)
         return FP8GEMM_E_SHAPE;
@@ -918,14 +992,17 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
     }
     if (live == 0)
         return FP8GEMM_OK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
     static_assert(GroupTable::MAX_GROUPS == FP8GEMM_MAX_GROUPS, "table size mirrors the ABI constant");
-    if (live <= GroupTable::MAX_GROUPS && g_selected.load() == FP8GEMM_KERNEL_AUTO && m_total <= 0x7FFFFFFFll) {
-        GroupTable tab;
-        tab.groups = 0;
+    if (live <= GroupTable::MAX_GROUPS && cfg.selected == FP8GEMM_KERNEL_AUTO && m_total <= 0x7FFFFFFFll) {
+        // Groups of at most 64 rows (an MoE layer in a decode step) go to the decode kernel, which streams
+        // every group's B once in whole lines; taller groups to the persistent tile kernel.  A pinned tile
+        // shape sends everything to the tile kernel.
+        GroupTable small, tall;
+        small.groups = tall.groups = 0;
         for (int g = 0; g < groups; ++g) {
             if (m[g] == 0)
                 continue;
+            GroupTable& tab = (m[g] <= 64 && cfg.force_variant < 0) ? small : tall;
             const int t = tab.groups++;
             tab.a[t] = static_cast<const uint8_t*>(a[g]);
             tab.b[t] = static_cast<const uint8_t*>(b[g]);
@@ -935,27 +1012,54 @@ int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* 
             tab.m[t] = m[g];
             tab.lda[t] = m[g];
         }
-        const int best_v = grouped_variant(tab, n, k);
-        if (best_v >= 0) {
-            const hipError_t e = launch_tile_grouped(tab, n, k, best_v, NUM_CU, s);
-            if (e == hipSuccess) {
-                snprintf(t_name_buf, sizeof(t_name_buf), "%s_k1_grouped%d", tile_variant_name(best_v), tab.groups);
-                t_last_kernel = t_name_buf;
-            }
-            return (int)e;
+        int rc = FP8GEMM_OK;
+        char first_name[sizeof(t_name_buf)] = "";
+        if (small.groups > 0) {
+            rc = run_grouped_table(small, n, k, true, s, cfg, explicit_ws);
+            if (rc == FP8GEMM_OK && tall.groups > 0)
+                snprintf(first_name, sizeof(first_name), "%s", t_name_buf);
         }
-        const int rc = run_grouped_padded(tab, n, k, s);
+        if (rc == FP8GEMM_OK && tall.groups > 0) {
+            rc = run_grouped_table(tall, n, k, false, s, cfg, explicit_ws);
+            if (rc == FP8GEMM_OK && first_name[0]) {  // both kernels ran: name both
+                char both[sizeof(t_name_buf)];
+                snprintf(both, sizeof(both), "%.28s+%.30s", first_name, t_name_buf);
+                snprintf(t_name_buf, sizeof(t_name_buf), "%s", both);
+            }
+        }
         if (rc != GROUPED_NOT_APPLICABLE)
             return rc;
+        // (a decode launch that already ran is simply run again below: same inputs, same outputs)
     }
     for (int g = 0; g < groups; ++g) {
         if (m[g] == 0)
             continue;
-        const int rc = run(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k, s, global_config(), nullptr);
+        const int rc = run(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k, s, cfg, explicit_ws);
         if (rc != FP8GEMM_OK)
             return rc;
     }
     return FP8GEMM_OK;
+}
+
+int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* b,
+                           const float* const* a_scale, const float* const* b_scale,
+                           void* const* c, const int* m, int n, int k, void* stream)
+{
+    return run_grouped(groups, a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), global_config(),
+                       nullptr);
+}
+
+int fp8_block_gemm_grouped_ex(int groups, const void* const* a, const void* const* b, const float* const* a_scale,
+                              const float* const* b_scale, void* const* c, const int* m, int n, int k,
+                              const fp8gemm_options* options, void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc;
+    const Config cfg = config_from_options(options, &rc);
+    if (rc != FP8GEMM_OK)
+        return rc;
+    const bool zeroed = options && (options->flags & FP8GEMM_FLAG_WORKSPACE_ZEROED) != 0;
+    const Workspace w{static_cast<float*>(workspace), workspace ? workspace_bytes : 0, zeroed};
+    return run_grouped(groups, a, b, a_scale, b_scale, c, m, n, k, static_cast<hipStream_t>(stream), cfg, &w);
 }
 
 int fp8_block_gemm_set_fused_reduction(int mode)
@@ -1007,30 +1111,43 @@ size_t fp8_block_gemm_workspace_bytes_ex(int m, int n, int k, const fp8gemm_opti
     return workspace_bytes_for(m, n, k, cfg, any_alignment != 0);
 }
 
-size_t fp8_block_gemm_grouped_workspace_bytes(int groups, const int* m, int n, int k)
+static size_t grouped_bytes(int groups, const int* m, int n, int k, const Config& cfg)
 {
     if (groups <= 0 || !m || n <= 0 || k <= 0 || (k % 128) != 0)
         return 0;
-    // the grouped launch on padded copies takes every group's copies at once; one by one the largest
-    // single need would do, which the sum covers
+    // a grouped launch on padded copies takes every group's copies at once (the decode kernel's splits meet
+    // in the header); one by one the largest single need would do
     const int n16 = (n + 15) & ~15;
     const size_t nkb = (size_t)k / 128;
-    size_t total = 0;
+    size_t total = 0, small_groups = 0;
     for (int g = 0; g < groups; ++g) {
         if (m[g] <= 0)
             continue;
         const size_t m16 = ((size_t)m[g] + 15) & ~(size_t)15;
         total += round256((size_t)k * m16) + round256(nkb * m16 * sizeof(float)) + round256((size_t)k * n16) +
                  round256(m16 * n16 * 2);
+        small_groups += m[g] <= 64 ? 1 : 0;
     }
-    total = with_header(total);
+    total = with_header(total, small_groups > 0);
     for (int g = 0; g < groups; ++g) {
         if (m[g] <= 0)
             continue;
-        const size_t single = workspace_bytes_for(m[g], n, k, global_config(), true);
+        const size_t single = workspace_bytes_for(m[g], n, k, cfg, true);
         total = total > single ? total : single;
     }
     return total;
+}
+
+size_t fp8_block_gemm_grouped_workspace_bytes(int groups, const int* m, int n, int k)
+{
+    return grouped_bytes(groups, m, n, k, global_config());
+}
+
+size_t fp8_block_gemm_grouped_workspace_bytes_ex(int groups, const int* m, int n, int k, const fp8gemm_options* options)
+{
+    int rc;
+    const Config cfg = config_from_options(options, &rc);
+    return rc == FP8GEMM_OK ? grouped_bytes(groups, m, n, k, cfg) : 0;
 }
 
 int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)
@@ -1142,6 +1259,6 @@ const char* fp8_block_gemm_error_string(int code)
 
 size_t fp8_block_gemm_workspace_growth(size_t have, size_t need) { return growth_target(have, need); }
 
-int fp8_block_gemm_abi_version(void) { return 4; }
+int fp8_block_gemm_abi_version(void) { return 5; }
 
 }  // extern "C"

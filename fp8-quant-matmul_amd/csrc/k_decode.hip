@@ -1,4 +1,4 @@
-// Wide-strip decode kernel for tiny M (M <= 32): HBM-bound, B is read exactly once, in whole
+// Wide-strip decode kernel for tiny M (M <= 64): HBM-bound, B is read exactly once, in whole
 // 128-byte lines.  The reference has no kernel for this regime (its smallest tile needs M >= 64,
 // /root/reference/mn_small.hip:16,121-125); the math is the same block-scaled product
 // (/root/reference/check.cu:36-48).
@@ -15,21 +15,31 @@
 // operands through ds_read_b64_tr_b8 as in the tile kernel): a wave ends with the complete partial
 // result of its 32 x 16 patch for the workgroup's K range and no reduction across waves is needed.
 //
-// The K splits of a strip are added inside the kernel, wave by wave, without a second launch:
+// The K splits of a strip are added inside the kernel, wave by wave, without a second launch and without
+// a ticket or a fence:
 //   * the workgroups of one strip are given linear ids that agree modulo 8, which the dispatcher
 //     places on one XCD (checked once per device by a probe grid, xcd_placement_confirmed): their
 //     stores and loads meet in that XCD's L2, and no device-scope fence -- a write-back of the whole
 //     L2 on this part -- is needed;
-//   * a wave stores its fp32 partial patch (register order, 1 KiB per instruction), waits for the
-//     stores' acknowledgement from L2 (s_waitcnt vmcnt(0)), and takes a ticket for (strip, wave) with
-//     a workgroup-scope atomic, which executes in that same L2;
-//   * the wave whose ticket says it arrived last loads all partial patches of its columns past its L1
-//     (sc0: a device-scope load, sc1, would also pass the L2 and cost a round trip to memory), adds them in split order -- the result does not depend on who arrived last -- and stores
-//     bf16.  The ticket wraps to zero with the last arrival (atomic inc with wrap), so the ticket
-//     words stay zero between launches; they must be zero before the first one.
+//   * the partial patches travel through a mailbox, a region of the workspace that only this kernel
+//     writes and that holds zeros whenever no launch is running.  A wave of every split but the last
+//     stores its fp32 partial patch there (register order, 1 KiB per instruction) with every +0.0 replaced
+//     by -0.0, so that no word it writes is zero, and is done: it waits for nothing;
+//   * the wave of the last split -- the workgroup with the highest id of its strip, dispatched after the
+//     others -- loads the patches of its 16 columns past its L1 (sc1) again and again until no word of
+//     them is zero, stores zeros back for the next launch, and adds them in split order, its own registers
+//     last: the sum does not depend on timing (adding -0.0 changes nothing, and a running sum that starts
+//     from +0.0 is never -0.0 itself).  A wave that has polled for a second gives up and writes NaN.
+// Against storing, waiting for the acknowledgement, taking a ticket with an atomic and loading as the last
+// arrival (three round trips to the L2, 2.8 us on the timeline of M = 32, N = 7168, K = 2048 split in
+// four) this is one store and the polling load.
+//
+// M <= 32 runs with two 16-row tiles of A (32-byte LDS rows), M <= 64 with four (64-byte rows); the same
+// body runs grouped problems (common N and K, own M <= 64, own operands: the experts of an MoE layer in a
+// decode step), whose strips form one list of work items.
 //
 // LDS stage: 128 k-rows x 128 B of B (chunk c of row r at position c ^ ((r >> 1) & 7)), 128 x 32 B
-// of A (chunk c at c ^ ((r >> 3) & 1)), the block's a_scale and b_scale values; six stages form a
+// of A (chunk c at c ^ ((r >> 3) & 1); 64-byte rows: c ^ ((r >> 2) & 3)), the block's a_scale and b_scale values; six stages form a
 // ring, up to five in flight while one is multiplied.  A CU takes in about 50 bytes per clock through
 // this path whatever the instruction mix, so the copy instructions of a workgroup's whole K range
 // (80 KB for a quarter of K = 2048) are what its run time is made of; small stages let the multiplying
@@ -46,17 +56,28 @@ namespace {
 
 constexpr int DS_BN = 128;
 constexpr int DS_THREADS = 512;
-constexpr int DS_MAT_B = KBLOCK * 128;
-constexpr int DS_MAT_A = KBLOCK * 32;
-constexpr int DS_SA_OFF = DS_MAT_B + DS_MAT_A;  // M floats (wave 4's copy)
-constexpr int DS_SB_OFF = DS_SA_OFF + 256;      // 1 float (wave 5's copy; waves 6 and 7 bring it again, 256 B apart)
-constexpr int DS_STAGE = DS_SB_OFF + 3 * 256;
 constexpr int DS_NS = 6;
-constexpr int DS_LDS = DS_NS * DS_STAGE;
-constexpr int DS_COPIES = 3;                    // copy instructions per wave and stage
-constexpr unsigned AUX_L1_MISS = 1;             // cache policy of the buffer loads (sc0): served by the L2
-static_assert(DS_LDS <= 160 * 1024, "ring exceeds the LDS");
-static_assert(DS_COPIES * (DS_NS - 2) < 64, "vmcnt is a 6-bit field");
+constexpr unsigned AUX_L1_MISS = 16;  // cache policy of the partial-patch loads (sc1): past the L1, served by the L2
+constexpr unsigned long long SPIN_LIMIT_TICKS = 100000000ull;  // one second of the constant 100 MHz counter (s_memrealtime)
+
+// MT = 16-row tiles of A a workgroup multiplies (2: M <= 32, 4: M <= 64)
+template <int MT>
+struct DecodeShape {
+    static constexpr int RSA = 16 * MT;                 // LDS bytes per k-row of A
+    static constexpr int MAT_B = KBLOCK * 128;
+    static constexpr int MAT_A = KBLOCK * RSA;
+    static constexpr int SA_OFF = MAT_B + MAT_A;        // up to 64 a_scale floats
+    static constexpr int SB_OFF = SA_OFF + 256;         // 1 float (every wave that brings it writes the same bytes)
+    static constexpr int STAGE = SB_OFF + 256;
+    static constexpr int LDS = DS_NS * STAGE;
+    // copy instructions per wave and stage: two of B, then A / scales
+    //   MT = 2: waves 0..3 A (32 rows x 32 B each), wave 4 a_scale, waves 5..7 b_scale
+    //   MT = 4: every wave A (16 rows x 64 B each), then wave 0 a_scale, waves 1..7 b_scale
+    static constexpr int COPIES = MT == 2 ? 3 : 4;
+    static_assert(MT == 2 || MT == 4, "two or four row tiles");
+    static_assert(LDS <= 160 * 1024, "ring exceeds the LDS");
+    static_assert(COPIES * (DS_NS - 2) < 64, "vmcnt is a 6-bit field");
+};
 
 template <int N>
 __device__ __forceinline__ void ds_wait_vmcnt()
@@ -64,12 +85,25 @@ __device__ __forceinline__ void ds_wait_vmcnt()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-__global__ void __launch_bounds__(DS_THREADS)
-decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
-                    const float* __restrict__ a_scale, const float* __restrict__ b_scale,
-                    uint16_t* __restrict__ c, float* __restrict__ partial, unsigned int* __restrict__ tickets,
-                    int M, int N, int K, int strips, int ksplit, int kb_per_split)
+// one problem as the kernel sees it
+struct DecodeProblem {
+    const uint8_t* a;
+    const uint8_t* b;
+    const float* a_scale;
+    const float* b_scale;
+    uint16_t* c;
+    int M;    // rows of c
+    int lda;  // elements between consecutive k-rows of a and of a_scale (>= M; rows M .. lda-1 hold zeros)
+};
+
+// Work units = (problem, strip), numbered problem-major; `units` of them.  Linear workgroup ids that
+// agree modulo 8 share an XCD: the ksplit workgroups of unit u sit at ids xcd + 8 * (grp * ksplit + split)
+// with u = grp * 8 + xcd.
+template <int MT, bool GROUPED>
+__device__ __forceinline__ void decode_body(const DecodeProblem& one, const GroupTable* tab, float* mailbox, int N, int K,
+                                            int strips, int units, int ksplit, int kb_per_split)
 {
+    using S = DecodeShape<MT>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     auto lds = LDS_PTR(uint8_t, smem);
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -77,28 +111,38 @@ decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
-    // linear ids that agree modulo 8 share an XCD: the ksplit workgroups of a strip sit at
-    // ids xcd + 8 * (group * ksplit + split)
     const int pid = blockIdx.x;
     const int xcd = pid & 7, j = pid >> 3;
     const int grp = j / ksplit, split = j - grp * ksplit;
-    const int strip = grp * 8 + xcd;
-    if (strip >= strips)
+    const int unit = grp * 8 + xcd;
+    if (unit >= units)
         return;
+    DecodeProblem pr = one;
+    int strip = unit;
+    if (GROUPED) {
+        const int g = unit / strips;
+        strip = unit - g * strips;
+        pr = DecodeProblem{tab->a[g], tab->b[g], tab->a_scale[g], tab->b_scale[g], tab->c[g], tab->m[g], tab->lda[g]};
+    }
+    const uint8_t* __restrict__ a = pr.a;
+    const uint8_t* __restrict__ b = pr.b;
+    const float* __restrict__ a_scale = pr.a_scale;
+    const float* __restrict__ b_scale = pr.b_scale;
+    uint16_t* __restrict__ c = pr.c;
+    const int M = pr.M, lda = pr.lda;
     const int n0 = strip * DS_BN;
 
     const int nkb = K / KBLOCK;
     const int kb0 = split * kb_per_split;
     const int kb1 = (kb0 + kb_per_split < nkb) ? (kb0 + kb_per_split) : nkb;
     const int sn = (N + KBLOCK - 1) / KBLOCK;
-    const int mtiles = (M + 15) >> 4;  // 1 or 2
+    const int mtiles = (M + 15) >> 4;  // 1 .. MT
 
-    // ---- copy plan, three instructions per wave and stage.  B: instruction q (0, 1) of a wave fills
-    // stage rows 16*wave + 8*q + (lane >> 3), chunk position lane & 7; the chunk swizzle (r >> 1) & 7 is
-    // (4*q + (lane >> 4)) & 7.  A: waves 0..3, rows 32*wave + (lane >> 1), position lane & 1, swizzle
-    // (r >> 3) & 1 = (lane >> 4) & 1.  Wave 4 brings the block's a_scale values, waves 5..7 its b_scale
-    // value (each into a slot of its own; wave 5's is read), so that every wave counts the same.
-    const uint32_t a_bytes = (uint32_t)M * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
+    // ---- copy plan.  B: instruction q (0, 1) of a wave fills stage rows 16*wave + 8*q + (lane >> 3), chunk
+    // position lane & 7; the chunk swizzle (r >> 1) & 7 is (4*q + (lane >> 4)) & 7.  A, 32-byte rows: waves
+    // 0..3, rows 32*wave + (lane >> 1), position lane & 1, swizzle (r >> 3) & 1 = (lane >> 4) & 1; 64-byte
+    // rows: every wave, rows 16*wave + (lane >> 2), position lane & 3, swizzle (r >> 2) & 3 = (lane >> 4) & 3.
+    const uint32_t a_bytes = (uint32_t)lda * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
     uint32_t voff_b[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
@@ -106,40 +150,42 @@ decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b
         const bool ok = n0 + 16 * cc < N;
         voff_b[q] = ok ? (uint32_t)((16 * wave + 8 * q + (lane >> 3)) * N + n0 + 16 * cc) : 0x80000000u;
     }
-    const int cca = (lane & 1) ^ ((lane >> 4) & 1);
-    uint32_t voff_3;  // the wave's third instruction
-    if (wave < 4)
-        voff_3 = 16 * cca < M ? (uint32_t)((32 * wave + (lane >> 1)) * M + 16 * cca) : 0x80000000u;
-    else if (wave == 4)
-        voff_3 = lane < M ? (uint32_t)(lane * 4) : 0x80000000u;
-    else
-        voff_3 = lane == 0 ? (uint32_t)(strip * 4) : 0x80000000u;
+    const uint32_t voff_sa = lane < lda ? (uint32_t)(lane * 4) : 0x80000000u;
+    const uint32_t voff_sb = lane == 0 ? (uint32_t)(strip * 4) : 0x80000000u;
+    uint32_t voff_a;
+    if (MT == 2) {
+        const int cc = (lane & 1) ^ ((lane >> 4) & 1);
+        voff_a = 16 * cc < lda ? (uint32_t)((32 * wave + (lane >> 1)) * lda + 16 * cc) : 0x80000000u;
+    } else {
+        const int cc = (lane & 3) ^ ((lane >> 4) & 3);
+        voff_a = 16 * cc < lda ? (uint32_t)((16 * wave + (lane >> 2)) * lda + 16 * cc) : 0x80000000u;
+    }
 
     // Stage `slot` <- K block kb.  The resources of A and B start at the block's first k-row.
     auto issue_stage = [&](int slot, int kb) __attribute__((always_inline)) {
-        const uint32_t stage = lds_base + (uint32_t)(slot * DS_STAGE);
+        const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
         const uint32_t skip_b = (uint32_t)kb * KBLOCK * (uint32_t)N;
+        const uint32_t skip_a = (uint32_t)kb * KBLOCK * (uint32_t)lda;
         const v4i rb = make_rsrc_words(b + skip_b, b_bytes - skip_b);
         lds_dma16(rb, voff_b[0], stage + (uint32_t)((2 * wave) * 1024));
         lds_dma16(rb, voff_b[1], stage + (uint32_t)((2 * wave + 1) * 1024));
-        if (wave < 4) {
-            const uint32_t skip_a = (uint32_t)kb * KBLOCK * (uint32_t)M;
-            lds_dma16(make_rsrc_words(a + skip_a, a_bytes - skip_a), voff_3, stage + DS_MAT_B + (uint32_t)(wave * 1024));
-        } else if (wave == 4) {
-            lds_dma4(make_rsrc_words(a_scale + (size_t)kb * M, (uint32_t)M * 4u), voff_3, stage + DS_SA_OFF);
-        } else {
-            lds_dma4(make_rsrc_words(b_scale + (size_t)kb * sn, (uint32_t)sn * 4u), voff_3,
-                     stage + DS_SB_OFF + (uint32_t)((wave - 5) * 256));
-        }
+        const int scale_wave = MT == 2 ? wave - 4 : wave;  // 0: a_scale, 1..: b_scale, below 0: A (two row tiles)
+        if (MT == 4 || wave < 4)
+            lds_dma16(make_rsrc_words(a + skip_a, a_bytes - skip_a), voff_a, stage + S::MAT_B + (uint32_t)(wave * 1024));
+        if (scale_wave == 0)
+            lds_dma4(make_rsrc_words(a_scale + (size_t)kb * lda, (uint32_t)lda * 4u), voff_sa, stage + S::SA_OFF);
+        else if (scale_wave > 0)
+            lds_dma4(make_rsrc_words(b_scale + (size_t)kb * sn, (uint32_t)sn * 4u), voff_sb, stage + S::SB_OFF);
     };
 
     // ---- transposing reads.  Lane = 16*g + i; read t of a K block covers k-rows 32*t + 8*g + (i >> 1),
-    // so (r >> 1) & 7 = (4*g + (i >> 2)) & 7 and (r >> 3) & 1 = g & 1 for every t and both blocks.
+    // so (r >> 1) & 7 = (4*g + (i >> 2)) & 7, (r >> 3) & 1 = g & 1 and (r >> 2) & 3 = (2*g + (i >> 3)) & 3
+    // for every t.
     const int g4 = lane >> 4, i16 = lane & 15;
     const uint32_t addr_b = (uint32_t)((8 * g4 + (i16 >> 1)) * 128 + ((wave ^ ((4 * g4 + (i16 >> 2)) & 7)) * 16) +
                                        (i16 & 1) * 8);
-    const uint32_t addr_a = (uint32_t)(DS_MAT_B + (8 * g4 + (i16 >> 1)) * 32 + (i16 & 1) * 8);
-    const uint32_t chunk_a[2] = {(uint32_t)((0 ^ (g4 & 1)) * 16), (uint32_t)((1 ^ (g4 & 1)) * 16)};
+    const uint32_t addr_a = (uint32_t)(S::MAT_B + (8 * g4 + (i16 >> 1)) * S::RSA + (i16 & 1) * 8);
+    const int swz_a = MT == 2 ? (g4 & 1) : ((2 * g4 + (i16 >> 3)) & 3);
     auto read_frag = [&](uint32_t addr, int step) __attribute__((always_inline)) -> v8i {
         v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr));
         v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr + step));
@@ -148,7 +194,10 @@ decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b
         return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
     };
 
-    v4f acc[2] = {(v4f){0.f, 0.f, 0.f, 0.f}, (v4f){0.f, 0.f, 0.f, 0.f}};
+    v4f acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+        acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int nstages = kb1 - kb0;
 #pragma unroll
@@ -162,22 +211,22 @@ decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b
         const int younger = nstages - 1 - s < DS_NS - 2 ? nstages - 1 - s : DS_NS - 2;
         switch (younger) {
         case 0: ds_wait_vmcnt<0>(); break;
-        case 1: ds_wait_vmcnt<DS_COPIES>(); break;
-        case 2: ds_wait_vmcnt<2 * DS_COPIES>(); break;
-        case 3: ds_wait_vmcnt<3 * DS_COPIES>(); break;
-        default: ds_wait_vmcnt<4 * DS_COPIES>(); break;
+        case 1: ds_wait_vmcnt<S::COPIES>(); break;
+        case 2: ds_wait_vmcnt<2 * S::COPIES>(); break;
+        case 3: ds_wait_vmcnt<3 * S::COPIES>(); break;
+        default: ds_wait_vmcnt<4 * S::COPIES>(); break;
         }
         __syncthreads();  // everyone's copies of stage s landed; the slot of stage s - 1 is no longer read
         if (s + DS_NS - 1 < nstages)
             issue_stage(slot == 0 ? DS_NS - 1 : slot - 1, kb0 + s + DS_NS - 1);
-        const uint32_t so = (uint32_t)(slot * DS_STAGE);
+        const uint32_t so = (uint32_t)(slot * S::STAGE);
         const v8i fb = read_frag(so + addr_b, 32 * 128);
-        const float sb = *LDS_PTR(float, lds + so + DS_SB_OFF);
+        const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < MT; ++i) {
             if (i < mtiles) {
-                const v8i fa = read_frag(so + addr_a + chunk_a[i], 32 * 32);
-                const float sa = *LDS_PTR(float, lds + so + DS_SA_OFF + (16 * i + i16) * 4);
+                const v8i fa = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
+                const float sa = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
                 const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                     fb, fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
                 const float sc = sa * sb;
@@ -190,9 +239,9 @@ decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b
 
     // ---- a lane holds C[16*i + (lane & 15)][n0 + 16*wave + 4*(lane >> 4) + 0..3]
     const int ncol = n0 + 16 * wave + 4 * g4;
-    auto store_c = [&](const v4f (&v)[2]) __attribute__((always_inline)) {
+    auto store_c = [&](const v4f (&v)[MT]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < MT; ++i) {
             const int mrow = 16 * i + i16;
             if (mrow < M && ncol < N) {
                 uint2 pk;
@@ -207,52 +256,100 @@ decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b
         return;
     }
 
-    // ---- this wave's partial patch, in register order: [strip][split][wave][i][lane] x 16 bytes
-    const size_t patch = ((size_t)(strip * ksplit) * 8 + wave) * 2;  // split 0; splits lie 16 patches apart
-    v4f* mine = reinterpret_cast<v4f*>(partial) + (patch + (size_t)split * 16) * 64 + lane;
-    mine[0] = acc[0];
-    mine[64] = acc[1];
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // acknowledged by the L2 this XCD's workgroups share
-    unsigned int ticket = 0;
-    if (lane == 0)
-        ticket = __builtin_amdgcn_atomic_inc32(tickets + strip * 8 + wave, (unsigned int)(ksplit - 1),
-                                               __ATOMIC_RELAXED, "workgroup");
-    ticket = (unsigned int)__builtin_amdgcn_readfirstlane((int)ticket);
-    if (ticket != (unsigned int)(ksplit - 1))
-        return;
-    // last to arrive for these 16 columns: every split's patch is in L2
-    const uint32_t span = (uint32_t)ksplit * 16u * 64u * 16u;  // bytes from this wave's split-0 patch to past its last
-    const __amdgpu_buffer_rsrc_t rp = make_rsrc(reinterpret_cast<const v4f*>(partial) + patch * 64, span);
-    // Every load goes out before the first sum.  A split past the last reads outside the resource, which
-    // fetches nothing.  (Taking this wave's own patch from its registers instead of loading it back was
-    // measured slower, 4 000 against 3 200 clocks for this phase.)
-    v4f sum[2] = {(v4f){0.f, 0.f, 0.f, 0.f}, (v4f){0.f, 0.f, 0.f, 0.f}};
-    auto gather = [&](auto nz_tag) __attribute__((always_inline)) {
-        constexpr int NZ = decltype(nz_tag)::value;
-        v4i v[NZ][2];
+    // ---- mailbox: [unit][split 0 .. ksplit-2][wave][i][lane] x 16 bytes, all zero between launches
+    constexpr int PER_SPLIT = 8 * MT;  // patches of one split of one unit
+    const int senders = ksplit - 1;
+    const size_t patch = ((size_t)unit * senders * 8 + wave) * MT;  // split 0
+    if (split < senders) {
+        v4i* mine = reinterpret_cast<v4i*>(mailbox) + (patch + (size_t)split * PER_SPLIT) * 64 + lane;
 #pragma unroll
-        for (int z = 0; z < NZ; ++z)
+        for (int i = 0; i < MT; ++i)
+            if (i < mtiles) {
+                v4i bits = __builtin_bit_cast(v4i, acc[i]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                v[z][i] = __builtin_amdgcn_raw_buffer_load_b128(rp, (uint32_t)((z * 16 + i) * 64 + lane) * 16u, 0,
-                                                                AUX_L1_MISS);
-#pragma unroll
-        for (int z = 0; z < NZ; ++z)
-            if (z < ksplit) {
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    const v4f f = __builtin_bit_cast(v4f, v[z][i]);
-                    sum[i] = z == 0 ? f : sum[i] + f;
-                }
+                for (int e = 0; e < 4; ++e)
+                    bits[e] = bits[e] == 0 ? (int)0x80000000 : bits[e];  // +0.0 -> -0.0: no word is zero
+                mine[64 * i] = bits;
             }
-    };
-    if (ksplit <= 4)
-        gather(std::integral_constant<int, 4>{});
-    else if (ksplit <= 8)
-        gather(std::integral_constant<int, 8>{});
-    else
-        gather(std::integral_constant<int, DECODE_MAX_KSPLIT>{});
+        return;
+    }
+    // last split: wait for the other splits' patches of these 16 columns, four splits at a time
+    const uint32_t span = (uint32_t)senders * PER_SPLIT * 64u * 16u;  // bytes from this wave's split-0 patch to past its last
+    const __amdgpu_buffer_rsrc_t rp = make_rsrc(reinterpret_cast<const v4i*>(mailbox) + patch * 64, span);
+    v4f sum[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+        sum[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    bool gave_up = false;
+    const unsigned long long t_first = __builtin_amdgcn_s_memrealtime();
+    for (int z0 = 0; z0 < senders; z0 += 4) {
+#pragma unroll
+        for (int h = 0; h < MT / 2; ++h) {  // two row tiles at a time
+            if (2 * h < mtiles) {
+                v4i v[4][2];
+                for (;;) {
+                    asm volatile("" ::: "memory");  // the loads belong to this round of the loop
+                    // a split past the last reads outside the resource, which fetches zeros
+#pragma unroll
+                    for (int z = 0; z < 4; ++z)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+                            v[z][i] = __builtin_amdgcn_raw_buffer_load_b128(
+                                rp, (uint32_t)(((z0 + z) * PER_SPLIT + 2 * h + i) * 64 + lane) * 16u, 0, AUX_L1_MISS);
+                    bool missing = false;
+#pragma unroll
+                    for (int z = 0; z < 4; ++z)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+                            if (z0 + z < senders && 2 * h + i < mtiles)
+                                missing = missing || v[z][i][0] == 0 || v[z][i][1] == 0 || v[z][i][2] == 0 || v[z][i][3] == 0;
+                    if (__builtin_amdgcn_ballot_w64(missing) == 0)
+                        break;
+                    if (__builtin_amdgcn_s_memrealtime() - t_first > SPIN_LIMIT_TICKS) {
+                        gave_up = true;
+                        break;
+                    }
+                }
+#pragma unroll
+                for (int z = 0; z < 4; ++z)
+                    if (z0 + z < senders) {
+#pragma unroll
+                        for (int i = 0; i < 2; ++i) {
+                            if (2 * h + i < mtiles)
+                                __builtin_amdgcn_raw_buffer_store_b128(
+                                    (v4i){0, 0, 0, 0}, rp, (uint32_t)(((z0 + z) * PER_SPLIT + 2 * h + i) * 64 + lane) * 16u, 0, 0);
+                            const v4f f = __builtin_bit_cast(v4f, v[z][i]);
+                            sum[2 * h + i] = z0 + z == 0 ? f : sum[2 * h + i] + f;
+                        }
+                    }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        sum[i] = sum[i] + acc[i];
+        if (gave_up)
+            sum[i] = (v4f){__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+    }
     store_c(sum);
+}
+
+template <int MT>
+__global__ void __launch_bounds__(DS_THREADS)
+decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
+                    const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int N, int K,
+                    int strips, int ksplit, int kb_per_split)
+{
+    const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
+    decode_body<MT, false>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
+}
+
+template <int MT>
+__global__ void __launch_bounds__(DS_THREADS)
+decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, int strips, int ksplit, int kb_per_split)
+{
+    const DecodeProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+    decode_body<MT, true>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
 }
 
 // records the XCC (XCD) id each workgroup of a probe grid runs on
@@ -267,28 +364,32 @@ __global__ void xcc_probe_kernel(unsigned int* out)
         out[blockIdx.x] = x & 0xFu;
 }
 
+inline int row_tiles(int m) { return m <= 32 ? 2 : 4; }
+
 }  // namespace
 
 bool decode_strip_supports(const GemmArgs& g)
 {
-    return g.m <= 32 && g.m % 16 == 0 && g.n % 16 == 0 && (g.lda == 0 || g.lda == g.m) &&
-           (g.n + DS_BN - 1) / DS_BN * 8 <= DECODE_TICKET_WORDS &&
+    return g.m <= 64 && g.m % 16 == 0 && g.n % 16 == 0 && (g.lda == 0 || g.lda == g.m) &&
            (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) && (reinterpret_cast<uintptr_t>(g.b) % 16 == 0) &&
-           (reinterpret_cast<uintptr_t>(g.a_scale) % 4 == 0) && (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
+           (reinterpret_cast<uintptr_t>(g.a_scale) % 4 == 0) && (reinterpret_cast<uintptr_t>(g.b_scale) % 4 == 0) &&
+           (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
 }
 
-size_t decode_strip_partial_bytes(const GemmArgs& g, int ksplit)
+// the mailbox of a K split: one patch per strip, sending split, wave and row tile
+bool decode_strip_can_split(const GemmArgs& g, int ksplit) { return decode_strip_mailbox_bytes(g, ksplit) <= DECODE_MAILBOX_BYTES; }
+
+size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit)
 {
     if (ksplit <= 1)
         return 0;
     const size_t strips = (size_t)(g.n + DS_BN - 1) / DS_BN;
-    return strips * (size_t)ksplit * 8 * 2 * 64 * 16;
+    return strips * (size_t)(ksplit - 1) * 8 * row_tiles(g.m) * 64 * 16;
 }
-
 // Microseconds with B streamed from HBM, fitted to M = 16 and 32, N = 1536 ... 16384, K = 1536 ... 7168 and
 // 1 to 16 K splits: a launch, then rounds of 256 workgroups, each workgroup living for a start-up, its
 // K blocks (0.5 us per block when few workgroups pull on HBM, 0.76 us when 256 do) and, when K is split,
-// the in-kernel reduction, whose last arrival reads one partial patch per split.
+// the in-kernel reduction, whose last split reads one partial patch per other split.
 double decode_strip_cost(const GemmArgs& g, int ksplit)
 {
     const int strips = (g.n + DS_BN - 1) / DS_BN;
@@ -332,20 +433,106 @@ int xcd_placement_confirmed(bool may_probe)
     return ok;
 }
 
-hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* partial, unsigned int* tickets, hipStream_t s)
+hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, hipStream_t s)
 {
     const int strips = (g.n + DS_BN - 1) / DS_BN;
     const int nkb = g.k / KBLOCK;
-    if (!decode_strip_supports(g) || ksplit < 1 || ksplit > nkb || ksplit > DECODE_MAX_KSPLIT || (ksplit > 1 && (!partial || !tickets)))
+    if (!decode_strip_supports(g) || ksplit < 1 || ksplit > nkb || ksplit > DECODE_MAX_KSPLIT ||
+        (ksplit > 1 && (!mailbox || !decode_strip_can_split(g, ksplit))))
         return hipErrorInvalidValue;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     if ((ksplit - 1) * kb_per_split >= nkb)  // every split owns at least one K block
         return hipErrorInvalidValue;
-    const int groups = (strips + 7) / 8;
-    auto kern = decode_strip_kernel;
-    FP8GEMM_ALLOW_LDS(kern, DS_LDS);
-    hipLaunchKernelGGL(kern, dim3(8 * groups * ksplit), dim3(DS_THREADS), DS_LDS, s, g.a, g.b, g.a_scale, g.b_scale,
-                       g.c, partial, tickets, g.m, g.n, g.k, strips, ksplit, kb_per_split);
+    const dim3 grid(8 * ((strips + 7) / 8) * ksplit);
+    if (row_tiles(g.m) == 2) {
+        auto kern = decode_strip_kernel<2>;
+        FP8GEMM_ALLOW_LDS(kern, DecodeShape<2>::LDS);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<2>::LDS, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
+                           mailbox, g.m, g.n, g.k, strips, ksplit, kb_per_split);
+    } else {
+        auto kern = decode_strip_kernel<4>;
+        FP8GEMM_ALLOW_LDS(kern, DecodeShape<4>::LDS);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<4>::LDS, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
+                           mailbox, g.m, g.n, g.k, strips, ksplit, kb_per_split);
+    }
+    return hipGetLastError();
+}
+
+// every group: 1 <= m <= lda <= 64 with lda a multiple of 16 (rows m .. lda-1 of a and a_scale hold zeros),
+// operands aligned like a single problem's
+bool decode_grouped_supports(const GroupTable& tab, int n, int k)
+{
+    if (tab.groups < 1 || tab.groups > GroupTable::MAX_GROUPS || k % KBLOCK != 0)
+        return false;
+    for (int g = 0; g < tab.groups; ++g) {
+        const GemmArgs ga{tab.a[g], tab.b[g], tab.a_scale[g], tab.b_scale[g], tab.c[g], tab.lda[g], n, k};
+        if (tab.m[g] <= 0 || tab.m[g] > tab.lda[g] || !decode_strip_supports(ga))
+            return false;
+    }
+    return true;
+}
+
+size_t decode_grouped_mailbox_bytes(const GroupTable& tab, int n, int ksplit)
+{
+    if (ksplit <= 1)
+        return 0;
+    int mmax = 0;
+    for (int g = 0; g < tab.groups; ++g)
+        mmax = tab.lda[g] > mmax ? tab.lda[g] : mmax;
+    const size_t units = (size_t)tab.groups * ((n + DS_BN - 1) / DS_BN);
+    return units * (size_t)(ksplit - 1) * 8 * row_tiles(mmax) * 64 * 16;
+}
+
+// the K split for a grouped launch: what the cost model picks for one problem with all the groups' strips
+// among the splits whose patches fit the mailbox; 1 when the in-kernel reduction cannot be used
+int decode_grouped_ksplit(const GroupTable& tab, int n, int k, bool fused_ok)
+{
+    const int strips = (n + DS_BN - 1) / DS_BN, nkb = k / KBLOCK;
+    const long units = (long)strips * tab.groups;
+    if (!fused_ok || units * DS_BN > 0x7FFFFFFFl)
+        return 1;
+    GemmArgs all{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], 32, (int)(units * DS_BN), k};
+    int best = 1;
+    double best_cost = decode_strip_cost(all, 1);
+    for (int ks = 2; ks <= DECODE_MAX_KSPLIT && ks <= nkb; ++ks) {
+        if ((ks - 1) * ((nkb + ks - 1) / ks) >= nkb || decode_grouped_mailbox_bytes(tab, n, ks) > DECODE_MAILBOX_BYTES)
+            continue;
+        const double cst = decode_strip_cost(all, ks);
+        if (cst < best_cost) {
+            best_cost = cst;
+            best = ks;
+        }
+    }
+    return best;
+}
+
+hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit, float* mailbox, hipStream_t s)
+{
+    const int strips = (n + DS_BN - 1) / DS_BN;
+    const int nkb = k / KBLOCK;
+    const long units = (long)strips * tab.groups;
+    if (!decode_grouped_supports(tab, n, k) || ksplit < 1 || ksplit > nkb || ksplit > DECODE_MAX_KSPLIT ||
+        units > 0x0FFFFFFF / DECODE_MAX_KSPLIT ||
+        (ksplit > 1 && (!mailbox || decode_grouped_mailbox_bytes(tab, n, ksplit) > DECODE_MAILBOX_BYTES)))
+        return hipErrorInvalidValue;
+    const int kb_per_split = (nkb + ksplit - 1) / ksplit;
+    if ((ksplit - 1) * kb_per_split >= nkb)
+        return hipErrorInvalidValue;
+    int mmax = 0;
+    for (int g = 0; g < tab.groups; ++g)
+        mmax = tab.lda[g] > mmax ? tab.lda[g] : mmax;
+    const dim3 grid((unsigned)(8 * ((units + 7) / 8) * ksplit));
+    if (row_tiles(mmax) == 2) {
+        auto kern = decode_strip_grouped_kernel<2>;
+        FP8GEMM_ALLOW_LDS(kern, DecodeShape<2>::LDS);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<2>::LDS, s, tab, mailbox, n, k, strips, ksplit,
+                           kb_per_split);
+    } else {
+        auto kern = decode_strip_grouped_kernel<4>;
+        FP8GEMM_ALLOW_LDS(kern, DecodeShape<4>::LDS);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<4>::LDS, s, tab, mailbox, n, k, strips, ksplit,
+                           kb_per_split);
+    }
     return hipGetLastError();
 }
 

@@ -86,15 +86,23 @@ int skinny_ksplit(const GemmArgs& g);
 double skinny_cost(const GemmArgs& g, int ksplit);
 hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStream_t s);
 
-// wide-strip decode kernel (M <= 32): 128-column strips, the K splits of a strip added inside the
-// kernel.  `partial` holds decode_strip_partial_bytes; `tickets` = DECODE_TICKET_WORDS words that are
-// zero before the launch and zero again after it.  ksplit > 1 needs xcd_placement_confirmed().
-constexpr int DECODE_TICKET_WORDS = TILE_TICKET_WORDS;
+// wide-strip decode kernel (M <= 64): 128-column strips, the K splits of a strip added inside the
+// kernel.  `mailbox` = DECODE_MAILBOX_BYTES of device memory that only this kernel writes, all zero before
+// the launch and all zero again after it (the splits hand their partial patches over through it).
+// ksplit > 1 needs xcd_placement_confirmed() and decode_strip_can_split.
+constexpr size_t DECODE_MAILBOX_BYTES = (size_t)8 << 20;
 constexpr int DECODE_MAX_KSPLIT = 16;
 bool decode_strip_supports(const GemmArgs& g);
-size_t decode_strip_partial_bytes(const GemmArgs& g, int ksplit);
+size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit);
+bool decode_strip_can_split(const GemmArgs& g, int ksplit);
 double decode_strip_cost(const GemmArgs& g, int ksplit);
-hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* partial, unsigned int* tickets, hipStream_t s);
+hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, hipStream_t s);
+// The same kernel on several problems with common n and k and their own m <= 64 (multiples of 16), whose
+// strips form one list of work items; tile_start of the table is not used.
+bool decode_grouped_supports(const GroupTable& tab, int n, int k);
+int decode_grouped_ksplit(const GroupTable& tab, int n, int k, bool fused_ok);
+size_t decode_grouped_mailbox_bytes(const GroupTable& tab, int n, int ksplit);
+hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit, float* mailbox, hipStream_t s);
 // 1 = workgroups whose linear ids agree modulo 8 share an XCD on the current device (looked at once
 // per device with a probe grid, which the first call waits for: not under stream capture),
 // 0 = they do not, or it could not be looked at; -1 = not looked at yet and may_probe is false

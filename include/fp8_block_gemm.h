@@ -107,10 +107,11 @@ int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 int fp8_block_gemm_set_persistent(int mode);
 
 /* Plans that split K ("..._kN") write fp32 partial results; they are added either by a second kernel or
- * inside the GEMM kernel by the workgroup (decode kernel: the wave) that finishes a tile last ("..._kNf",
- * "decode128_kN"): the K splits of a tile are placed on one XCD, meet in its L2 and count themselves in
- * with a ticket, and the last arrival adds the partials in split order, so the result does not depend on
- * who is last and equals the second kernel's bit for bit.  mode -1 = by cost (default), 0 = never,
+ * inside the GEMM kernel ("..._kNf", "decode128_kN"): the K splits of a tile are placed on one XCD and meet
+ * in its L2.  Tile kernels count themselves in with a ticket and the workgroup that finishes a tile last adds
+ * the partials in split order, so the result does not depend on who is last and equals the second kernel's
+ * bit for bit; in the decode kernel the waves of the last split poll a zero-initialised mailbox for the other
+ * splits' partial patches and add them in split order (a wave that polls for a second writes NaN).  mode -1 = by cost (default), 0 = never,
  * 1 = whenever the plan allows.  The first call that could use it on a device looks once at where that
  * device places workgroups (a probe grid the call waits for; skipped, and the two-kernel form used, while
  * the stream is being captured and the answer is not known yet).  The reference does not split K
@@ -125,9 +126,14 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * run as ONE launch of the persistent tile kernel (their tiles form one list that 256
  * workgroups walk through): as they are when every m[g] and n are multiples of 16 and the
  * operands 16-byte aligned, else on zero-padded copies in the workspace made by one batched copy
- * launch per operand kind ("padded_..._groupedN").  More groups than that fall back to one call
+ * launch per operand kind ("padded_..._groupedN").  Groups of at most 64 rows (the experts of an MoE
+ * layer in a decode step) do not go through 128-row tiles: they run as ONE launch of the decode kernel
+ * ("decode128_kN_groupedG": 128-column strips of every group in one work list, every group's B read
+ * once, the K range split and added inside the kernel as for a single problem); a call that mixes both
+ * kinds launches each kernel once.  More groups than FP8GEMM_MAX_GROUPS fall back to one call
  * of fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to
- * what fp8_block_gemm_stream gives for that problem with the same tile shape.  No counterpart in the
+ * what fp8_block_gemm_stream gives for that problem with the same tile shape (decode kernel: with the
+ * same K split).  No counterpart in the
  * reference, which launches one problem at a time (/root/reference/check.cu:106-114). */
 #define FP8GEMM_MAX_GROUPS 64
 int fp8_block_gemm_grouped(int groups, const void* const* a, const void* const* b,
@@ -150,12 +156,13 @@ typedef struct fp8gemm_options {
 } fp8gemm_options;
 /* The first FP8GEMM_WORKSPACE_HEADER_BYTES of the workspace handed to this call were zero-filled by the
  * caller before the first call that used this workspace, and nothing but this library has written to the
- * workspace since.  The library keeps arrival tickets there (zero again after every call) for the plans
- * that add the K splits of a tile or strip inside the GEMM kernel instead of launching a reduction kernel
- * ("decode128_kN", "..._kNf"); without the flag a per-call workspace only gets the two-kernel plans.
- * The process-wide workspace and fp8_block_gemm_noalloc's array always have zeroed tickets. */
+ * workspace since.  The plans that add the K splits of a tile or strip inside the GEMM kernel instead of
+ * launching a reduction kernel ("decode128_kN", "..._kNf") keep their hand-over state there -- arrival
+ * tickets (16 KiB) and the decode kernel's mailbox of partial patches (8 MiB) -- and leave all of it zero
+ * again after every call; without the flag a per-call workspace only gets the two-kernel plans.
+ * The process-wide workspace and fp8_block_gemm_noalloc's array always have a zeroed header. */
 #define FP8GEMM_FLAG_WORKSPACE_ZEROED 1
-#define FP8GEMM_WORKSPACE_HEADER_BYTES 16384
+#define FP8GEMM_WORKSPACE_HEADER_BYTES (16384 + (8u << 20))
 int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
                       int m, int n, int k, const fp8gemm_options* options, void* workspace,
                       size_t workspace_bytes, void* stream);
@@ -169,6 +176,20 @@ int fp8_block_gemm_ws(const void* a, const void* b, const float* a_scale, const 
  * Touches no device.  0 for an invalid shape or options. */
 size_t fp8_block_gemm_workspace_bytes_ex(int m, int n, int k, const fp8gemm_options* options,
                                          int any_alignment);
+/* Per-call form of fp8_block_gemm_grouped: same arguments and results, with `options` and `workspace`
+ * as for fp8_block_gemm_ex (nothing process-wide is read or written, nothing is allocated; safe from
+ * several host threads on several streams with distinct workspaces, and under stream capture).
+ * fp8_block_gemm_grouped_workspace_bytes_ex bounds the workspace for any alignment of the operands;
+ * with less than that (or none) the groups that need a workspace run one by one, or the call returns
+ * FP8GEMM_E_WORKSPACE when a single group needs more than it was given.  The decode kernel splits K
+ * only with FP8GEMM_FLAG_WORKSPACE_ZEROED.  No counterpart in the reference (one problem at a time on
+ * stream 0, /root/reference/check.cu:106-119). */
+int fp8_block_gemm_grouped_ex(int groups, const void* const* a, const void* const* b,
+                              const float* const* a_scale, const float* const* b_scale, void* const* c,
+                              const int* m, int n, int k, const fp8gemm_options* options, void* workspace,
+                              size_t workspace_bytes, void* stream);
+size_t fp8_block_gemm_grouped_workspace_bytes_ex(int groups, const int* m, int n, int k,
+                                                 const fp8gemm_options* options);
 
 /* fp8_block_gemm_stream for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): the same dispatch under the same process-wide switches, but

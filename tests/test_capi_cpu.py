@@ -14,7 +14,7 @@ def test_library_exports_every_declared_symbol(pkg):
     assert len(names) >= 22
     for name in names:
         assert hasattr(L, name), f"{name} declared in the header but not exported"
-    assert L.fp8_block_gemm_abi_version() == 4
+    assert L.fp8_block_gemm_abi_version() == 5
 
 
 def test_argument_validation_happens_before_any_device_call(pkg):
@@ -59,6 +59,18 @@ def test_grouped_entry_point_validates_every_group_first(pkg):
     assert L.fp8_block_gemm_grouped(2, ok, ok, ok, ok, ok, ints(16, -4), 16, 128, None) == -2
     with pytest.raises(ValueError):
         pkg.gemm_grouped([p], [p, p], [p], [p], [p], [16], 16, 128)
+    # the per-call form validates the same way, and its options as fp8_block_gemm_ex does
+    ex = L.fp8_block_gemm_grouped_ex
+    assert ex(-1, ok, ok, ok, ok, ok, ints(16, 16), 16, 128, None, None, 0, None) == -2
+    assert ex(2, ok, ok, ok, ok, ok, None, 16, 128, None, None, 0, None) == -1
+    assert ex(2, ok, ok, ok, ok, ok, ints(0, 0), 16, 128, None, None, 0, None) == 0
+    assert ex(2, ok, arr(p, None), ok, ok, ok, ints(16, 16), 16, 128, None, None, 0, None) == -1
+    assert ex(2, ok, ok, ok, ok, ok, ints(16, -4), 16, 128, None, None, 0, None) == -2
+    bad = pkg.Options(kernel=9)
+    assert ex(2, ok, ok, ok, ok, ok, ints(16, 16), 16, 128, C.byref(bad), None, 0, None) == \
+        L.fp8_block_gemm_ex(p, p, p, p, p, 16, 16, 128, C.byref(bad), None, 0, None) != 0
+    with pytest.raises(ValueError):
+        pkg.gemm_grouped_ex([p], [p, p], [p], [p], [p], [16], 16, 128)
 
 
 def test_error_strings_and_exception(pkg):
@@ -155,6 +167,13 @@ def test_workspace_queries_cover_every_alignment(pkg):
     assert tot >= sum(2048 * ((x + 15) // 16 * 16) for x in ms)
     assert tot >= max(pkg.workspace_bytes_ex(x, 7168, 2048, None, True) for x in ms)
     assert pkg.grouped_workspace_bytes([], 7168, 2048) == 0
+    # decode-sized groups: the header (their K splits meet in its mailbox) and every group's padded copies
+    small = [16, 64, 33]
+    assert pkg.grouped_workspace_bytes(small, 7168, 2048) >= pkg.WORKSPACE_HEADER_BYTES + sum(
+        2048 * ((x + 15) // 16 * 16) + 2048 * 7168 for x in small)
+    assert pkg.grouped_workspace_bytes([16, 32], 256, 256) >= pkg.WORKSPACE_HEADER_BYTES
+    assert pkg.grouped_workspace_bytes(small, 7168, 2048, per_call=True) == pkg.grouped_workspace_bytes(small, 7168, 2048)
+    assert pkg.grouped_workspace_bytes(small, 7168, 2048, pkg.Options(kernel=9)) == 0
 
 
 def test_noalloc_entry_point_validates_before_any_device_call(pkg):
@@ -205,7 +224,7 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(16, 1536, 2048) == "decode128_k4"
     assert pkg.plan(32, 16384, 7168) == "decode128_k2"     # 128 strips x 2
     assert pkg.plan(32, 128, 128) == "decode128_k1"        # one K block: nothing to split
-    assert pkg.workspace_bytes(32, 7168, 2048) == pkg.WORKSPACE_HEADER_BYTES + 56 * 4 * 16384
+    assert pkg.workspace_bytes(32, 7168, 2048) == pkg.WORKSPACE_HEADER_BYTES   # the splits meet in the header's mailbox
     assert pkg.plan(64, 1536, 7168) == "tile64x64_k7f"     # a single row of tiles: never fewer than 8 K blocks per split
     assert pkg.plan(48, 1536, 1536) == "tile64x64_k1"
     pkg.select(pkg.KERNEL_SKINNY)

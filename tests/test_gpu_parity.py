@@ -234,13 +234,13 @@ def test_skinny_kernel_with_the_k_range_split_over_workgroups(pkg, m, n, k, kspl
     _assert_every_element(got, a, b, sa, sb, m, n, k, name)
 
 
-# wide strips (128 columns), the K splits of a strip added inside the kernel by the last wave to arrive:
+# wide strips (128 columns), the K splits of a strip added inside the kernel by the waves of its last split:
 # every K split count the kernel takes, one and two row tiles, a ragged last strip (n % 128 != 0), more
 # strips x splits than CUs (several rounds of workgroups), a single K block per split
 DECODE_STRIP_CASES = [(32, 7168, 2048, 4), (16, 7168, 2048, 4), (32, 7168, 2048, 1), (32, 576, 1024, 3),
                       (32, 1040, 2048, 16), (16, 96, 512, 2), (32, 128, 128, 1), (32, 4608, 7168, 7),
-                      (16, 1536, 1536, 12), (32, 2048, 384, 3), (32, 16384, 1024, 8), (16, 16, 2048, 6),
-                      (32, 7168, 7168, 14)]
+                      (16, 1536, 1536, 12), (32, 2048, 384, 3), (32, 16384, 1024, 4), (16, 16, 2048, 6),
+                      (32, 7168, 7168, 8)]
 
 
 @pytest.mark.parametrize("m,n,k,ksplit", DECODE_STRIP_CASES)
@@ -251,14 +251,23 @@ def test_decode_strip_kernel(pkg, m, n, k, ksplit):
     assert name == f"decode128_k{ksplit}", name
     _assert_close(got, ref, name)
     _assert_every_element(got, a, b, sa, sb, m, n, k, name)
-    # the sum runs in split order whoever arrives last, and the tickets are zero again after every launch
+    # the sum runs in split order whatever the timing, and the mailbox is zero again after every launch
     for rep in range(4):
         again, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ksplit)
         assert np.array_equal(got, again), f"run {rep}: not reproducible"
 
 
-def test_decode_strip_tickets_survive_a_change_of_shape(pkg):
-    """launches of different strip and split counts back to back share the ticket words"""
+def test_decode_strip_split_that_outgrows_the_mailbox_is_refused(pkg):
+    """128 strips x 7 sending splits x 16 KiB of patches do not fit the 8 MiB mailbox: no such plan"""
+    m, n, k = 32, 16384, 1024
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1290)
+    with pytest.raises(pkg.Fp8GemmError) as info:
+        _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=8)
+    assert info.value.code == -3
+
+
+def test_decode_strip_mailbox_survives_a_change_of_shape(pkg):
+    """launches of different strip and split counts back to back share the mailbox"""
     import torch
     st = torch.cuda.current_stream().cuda_stream
     cases = [(32, 7168, 2048, 4), (16, 1536, 1024, 8), (32, 7168, 2048, 2), (32, 640, 4096, 16), (32, 7168, 2048, 4)]
@@ -283,9 +292,9 @@ def test_decode_strip_tickets_survive_a_change_of_shape(pkg):
 
 
 def test_decode_strips_in_a_caller_workspace_need_its_zeroed_flag(pkg):
-    """fp8_block_gemm_ex: the in-kernel reduction keeps tickets at the start of the workspace, so a per-call
-    workspace gets it only when the caller vouches for zeroed ticket words; without the flag the call
-    takes a plan that needs none"""
+    """fp8_block_gemm_ex: the in-kernel reduction keeps its hand-over state (tickets, the decode kernel's
+    mailbox) in the header of the workspace, so a per-call workspace gets it only when the caller vouches for
+    a zeroed header; without the flag the call takes a plan that needs none"""
     import torch
     m, n, k = 32, 7168, 2048
     a, b, sa, sb = oracle.make_inputs(m, n, k, 1400)
@@ -293,8 +302,8 @@ def test_decode_strips_in_a_caller_workspace_need_its_zeroed_flag(pkg):
     dev = _dev(a, b, sa, sb)
     st = torch.cuda.current_stream().cuda_stream
     need = pkg.workspace_bytes_ex(m, n, k)
-    assert need == pkg.WORKSPACE_HEADER_BYTES + 56 * 4 * 16384
-    ws = torch.full((need,), 0xAB, dtype=torch.uint8, device="cuda")          # garbage, also in the ticket words
+    assert need == pkg.WORKSPACE_HEADER_BYTES
+    ws = torch.full((need,), 0xAB, dtype=torch.uint8, device="cuda")          # garbage, also in the header
     dc = torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)
     _say(f"[gpu case] decode in a caller workspace without / with the zeroed flag m={m} n={n} k={k}")
     pkg.gemm_ex(dev[0], dev[1], dev[2], dev[3], dc, m, n, k, None, ws, need, st)
@@ -309,7 +318,7 @@ def test_decode_strips_in_a_caller_workspace_need_its_zeroed_flag(pkg):
     torch.cuda.synchronize()
     assert pkg.last_kernel() == "decode128_k4", pkg.last_kernel()
     _assert_close(dc.cpu().numpy().view(np.uint16), ref, "decode128_k4 in a caller workspace")
-    assert int(ws[:pkg.WORKSPACE_HEADER_BYTES].to(torch.int32).sum().item()) == 0, "tickets not back to zero"
+    assert int(ws[:pkg.WORKSPACE_HEADER_BYTES].to(torch.int32).sum().item()) == 0, "header not back to zero"
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 7168, 7168), (16, 4608, 7168), (32, 1536, 7168), (32, 7168, 4096),
@@ -636,7 +645,11 @@ def test_grouped_gemm_pads_groups_off_the_16_byte_grid(pkg, ms, n, k):
                      outs, ms, n, k, st)
     torch.cuda.synchronize()
     name = pkg.last_kernel()
-    assert name.startswith("padded_") and name.endswith(f"_grouped{sum(1 for m in ms if m)}"), name
+    # groups of at most 64 rows go to the decode kernel, taller ones to the tile kernel: one launch of each
+    parts = name.split("+")
+    assert any(p.startswith("padded_") for p in parts), name           # each launch pads only if its own groups need it
+    assert sum(int(p.rsplit("_grouped", 1)[1]) for p in parts) == sum(1 for m in ms if m), name
+    assert ("decode128" in name) == any(0 < m <= 64 for m in ms) and ("tile" in name) == any(m > 64 for m in ms), name
     for g, m in enumerate(ms):
         got = outs[g].cpu().numpy().view(np.uint16)
         assert (got[m:] == 0x7FC1).all(), f"group {g}: rows beyond m written"
@@ -665,6 +678,60 @@ def test_grouped_gemm_takes_more_groups_than_one_launch_holds(pkg):
     for g, m in enumerate(ms):
         a, b, sa, sb = host[g]
         _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
+    pkg.release()
+
+
+@pytest.mark.parametrize("ms,n,k", [([16, 32, 64, 48, 16, 0, 32], 1536, 2048),      # K split inside the kernel
+                                    ([64] * 24, 512, 1024),
+                                    ([16] * 64, 256, 384),
+                                    ([32, 48], 576, 128),                             # one K block: nothing to split
+                                    ([16, 64, 32, 16], 7168, 512)])
+def test_grouped_decode_groups_equal_the_problems_one_by_one(pkg, ms, n, k):
+    """groups of at most 64 rows (an MoE layer in a decode step): one launch of the decode kernel, every
+    group bit-identical to a single launch of that kernel with the same K split"""
+    host, dev, outs, name = _grouped_case(pkg, ms, n, k, -1, 9100 + n + k)
+    live = sum(1 for m in ms if m)
+    assert name.startswith("decode128_k") and name.endswith(f"_grouped{live}"), name
+    ks = int(name.split("_k")[1].split("_")[0])
+    for g, m in enumerate(ms):
+        if m == 0:
+            assert (outs[g].cpu().numpy().view(np.uint16) == 0x7FC1).all()      # untouched
+            continue
+        a, b, sa, sb = host[g]
+        got = outs[g].cpu().numpy().view(np.uint16)
+        _assert_close(got, oracle.ref_gemm(a, b, sa, sb, m, n, k), f"{name} group {g}")
+        _assert_every_element(got, a, b, sa, sb, m, n, k, f"{name} group {g}")
+        single, sname = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ks)
+        assert sname == f"decode128_k{ks}", sname
+        assert np.array_equal(got, single), f"group {g}: grouped launch and single launch differ"
+
+
+def test_grouped_decode_groups_off_the_16_byte_grid_and_mixed_with_tall_groups(pkg):
+    """ragged token counts of 1 to 64 rows run on padded copies in one decode launch; a call that also holds
+    taller groups launches the tile kernel for those; rows beyond m stay untouched"""
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    for ms, n, k in [([1, 7, 64, 33, 16, 50, 2], 1536, 1024), ([5, 300, 64, 1000, 17], 640, 512), ([3, 9], 200, 256)]:
+        host, dev, outs = [], [], []
+        for g, m in enumerate(ms):
+            a, b, sa, sb = oracle.make_inputs(m, n, k, 9300 + 11 * g + n)
+            host.append((a, b, sa, sb))
+            dev.append(_dev(a, b, sa, sb))
+            outs.append(torch.full((m + 16, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16))
+        _say(f"[gpu case] grouped decode, ragged ms={ms} n={n} k={k}")
+        pkg.gemm_grouped([d[0] for d in dev], [d[1] for d in dev], [d[2] for d in dev], [d[3] for d in dev],
+                         outs, ms, n, k, st)
+        torch.cuda.synchronize()
+        name = pkg.last_kernel()
+        assert "decode128_k" in name and name.startswith("padded_"), name
+        if max(ms) > 64:
+            assert "+" in name and "tile" in name, name
+        for g, m in enumerate(ms):
+            got = outs[g].cpu().numpy().view(np.uint16)
+            assert (got[m:] == 0x7FC1).all(), f"group {g}: rows beyond m written"
+            a, b, sa, sb = host[g]
+            _assert_close(got[:m], oracle.ref_gemm(a, b, sa, sb, m, n, k), f"{name} group {g}")
+            _assert_every_element(got[:m], a, b, sa, sb, m, n, k, f"{name} group {g}")
     pkg.release()
 
 

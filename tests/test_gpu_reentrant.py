@@ -231,3 +231,83 @@ def test_library_owned_workspace_growth_keeps_device_memory_bounded(pkg):
         pkg.select(0)
         pkg.force_config(-1, 0)
     pkg.release()
+
+
+def test_grouped_per_call_form_from_two_threads_on_two_streams(pkg):
+    """fp8_block_gemm_grouped_ex: two grouped calls (decode-sized groups with the K range split inside the
+    kernel; ragged taller groups on padded copies) run at the same time, each on its own stream with its own
+    zeroed workspace; results equal the ones each call gives alone and the oracle's."""
+    import torch
+    jobs = []
+    for (ms, n, k, seed) in [([16, 64, 32, 48, 16, 16, 64, 32], 1536, 2048, 8601), ([250, 40, 1000], 392, 512, 8602)]:
+        host, dev = [], []
+        for g, m in enumerate(ms):
+            a, b, sa, sb = oracle.make_inputs(m, n, k, seed + 31 * g)
+            host.append((a, b, sa, sb))
+            dev.append(_dev(a, b, sa, sb))
+        opt = pkg.Options(flags=pkg.FLAG_WORKSPACE_ZEROED)
+        need = pkg.grouped_workspace_bytes(ms, n, k, opt)
+        assert need > pkg.WORKSPACE_HEADER_BYTES
+        jobs.append(dict(ms=ms, n=n, k=k, host=host, dev=dev, opt=opt, need=need,
+                         ws=torch.zeros(need, dtype=torch.uint8, device="cuda"),
+                         outs=[torch.zeros((m, n), dtype=torch.int16, device="cuda") for m in ms],
+                         stream=torch.cuda.Stream()))
+    torch.cuda.synchronize()
+
+    def call(j):
+        d = j["dev"]
+        pkg.gemm_grouped_ex([x[0] for x in d], [x[1] for x in d], [x[2] for x in d], [x[3] for x in d], j["outs"],
+                            j["ms"], j["n"], j["k"], j["opt"], j["ws"], j["need"], j["stream"].cuda_stream)
+
+    for j in jobs:
+        _say(f"[gpu case] grouped per-call entry point alone ms={j['ms']}")
+        call(j)
+        torch.cuda.synchronize()
+        j["name"] = pkg.last_kernel()
+        j["alone"] = [c.cpu().numpy().copy() for c in j["outs"]]
+        for g, m in enumerate(j["ms"]):
+            ref = oracle.ref_gemm(*j["host"][g], m, j["n"], j["k"])
+            assert oracle.compare_bf16(j["alone"][g].view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0, (j["name"], g)
+    assert jobs[0]["name"].startswith("decode128_k") and not jobs[0]["name"].startswith("decode128_k1_"), jobs[0]["name"]
+    assert "padded_" in jobs[1]["name"] and "+" in jobs[1]["name"], jobs[1]["name"]
+    errors = []
+
+    def worker(j, rounds):
+        try:
+            for _ in range(rounds):
+                call(j)
+        except Exception as exc:
+            errors.append(exc)
+
+    _say("[gpu case] grouped per-call entry point from two threads on two streams")
+    for j in jobs:
+        for c in j["outs"]:
+            c.fill_(-1)
+    torch.cuda.synchronize()
+    threads = [threading.Thread(target=worker, args=(j, 100)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for j in jobs:
+        for g in range(len(j["ms"])):
+            assert np.array_equal(j["outs"][g].cpu().numpy(), j["alone"][g]), (j["ms"], g)
+    # without a workspace the decode-sized groups still run as one launch, unsplit; ragged groups cannot
+    j = jobs[0]
+    d = j["dev"]
+    pkg.gemm_grouped_ex([x[0] for x in d], [x[1] for x in d], [x[2] for x in d], [x[3] for x in d], j["outs"],
+                        j["ms"], j["n"], j["k"], None, None, 0, j["stream"].cuda_stream)
+    torch.cuda.synchronize()
+    assert pkg.last_kernel() == f"decode128_k1_grouped{len(j['ms'])}", pkg.last_kernel()
+    for g, m in enumerate(j["ms"]):
+        ref = oracle.ref_gemm(*j["host"][g], m, j["n"], j["k"])
+        assert oracle.compare_bf16(j["outs"][g].cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0
+    j = jobs[1]
+    d = j["dev"]
+    with pytest.raises(pkg.Fp8GemmError) as info:
+        pkg.gemm_grouped_ex([x[0] for x in d], [x[1] for x in d], [x[2] for x in d], [x[3] for x in d], j["outs"],
+                            j["ms"], j["n"], j["k"], None, None, 0, j["stream"].cuda_stream)
+    assert info.value.code == -4
+    torch.cuda.synchronize()
