@@ -15,7 +15,7 @@ _LIB = None
 KERNEL_AUTO, KERNEL_SCALAR, KERNEL_LARGE, KERNEL_SPLITK, KERNEL_SKINNY = range(5)
 DTYPE_BF16, DTYPE_F32, DTYPE_BF16_F32MATH = 0, 1, 2
 FLAG_WORKSPACE_ZEROED = 1
-WORKSPACE_HEADER_BYTES = 16384 + (8 << 20)
+WORKSPACE_HEADER_BYTES = 16 << 20
 
 
 class Options(C.Structure):

@@ -50,19 +50,17 @@ constexpr int MAX_KSPLIT = 16;
 // device memory a call may use beyond its operands: fp32 partial sums of plans that split K, padded
 // copies of operands off the 16-byte grid
 // The first WS_HEADER bytes belong to the kernels that add their K splits themselves and are zero before
-// the first call and after every call: the arrival tickets of the tile kernels, then the mailbox through
-// which the decode kernel's splits hand over their partial patches.  Plans keep their data behind it.
+// the first call and after every call: the mailbox through which the splits of a tile or strip hand over
+// their partial results.  Plans keep their data behind it.
 struct Workspace {
     float* ptr;
     size_t bytes;
     bool zeroed;  // the header was zero-filled when the buffer was taken on and only this library wrote to it since
 };
-constexpr size_t WS_TICKET_BYTES = (size_t)TILE_TICKET_WORDS * sizeof(unsigned int);
-constexpr size_t WS_HEADER = WS_TICKET_BYTES + DECODE_MAILBOX_BYTES;
+constexpr size_t WS_HEADER = SPLIT_MAILBOX_BYTES;
 static_assert(WS_HEADER == FP8GEMM_WORKSPACE_HEADER_BYTES, "the header size is part of the ABI");
 inline float* ws_data(const Workspace& w) { return w.ptr ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(w.ptr) + WS_HEADER) : nullptr; }
-inline unsigned int* ws_tickets(const Workspace& w) { return reinterpret_cast<unsigned int*>(w.ptr); }
-inline float* ws_mailbox(const Workspace& w) { return w.ptr ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(w.ptr) + WS_TICKET_BYTES) : nullptr; }
+inline float* ws_mailbox(const Workspace& w) { return w.ptr; }
 
 std::mutex g_ws_mutex;
 float* g_ws_own = nullptr;       // library-owned workspace
@@ -160,7 +158,7 @@ int validate(const void* a, const void* b, const float* as, const float* bs, con
 // least-squares fit to a sweep of every tile variant x ksplit over the 18 shapes of the
 // reference's table (/root/reference/README.md:15-25) and the five benchmark shapes (rms
 // error 10 %, the chosen plan within 6 % of the best measured one on all of them).
-double tile_cost(const GemmArgs& g, int variant, int ksplit)
+double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
 {
     int bm, bn;
     tile_variant_dims(variant, &bm, &bn);
@@ -178,20 +176,36 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit)
     const long slots = (variant == TILE_64x64 && g.m <= 64) ? 2 * NUM_CU : NUM_CU;
     const long rounds = (items + slots - 1) / slots;
     double cost = 1.79 + rounds * per_item;
-    if (ksplit > 1)  // second launch + partial write and read-back
+    if (ksplit > 1 && fused)  // the last split of a tile waits for the others' accumulators and reads them
+        cost += 1.8 + 0.35 * (ksplit - 1) * (double)(bm * bn) / 4096.0;
+    else if (ksplit > 1)  // second launch + partial write and read-back
         cost += 2.86 + (double)g.m * g.n * ksplit * 8.0 / 7.38e6;
     return cost;
 }
 
 // The in-kernel reduction against the reduction kernel, measured on 11 shapes x 13 split plans (all
-// bit-identical): the last workgroup of a tile reads ksplit partial tiles at the 15-20 bytes per clock
-// one CU takes in, so it pays while that is little -- 64x64 tiles (16 KB per split): 2-30 % faster up
-// to 4 splits, even at 8 -- and loses from 128x128 tiles on (64 KB per split: +2 ... +40 %; 256x192:
-// up to 3 x), where the reduction kernel's 256 CUs read the partials together.
+// bit-identical): the workgroup of a tile's last split reads the other splits' accumulators at the 15-20
+// bytes per clock one CU takes in, so it pays while that is little -- 64x64 tiles (16 KB per split): 2-35 %
+// faster up to 8 splits; 128x128 tiles (64 KB per split): 0-45 % faster with two or three splits unless
+// only a handful of workgroups run (256 x 256 x 7168: 2-6 % slower) -- and loses beyond (128x128 with six
+// splits +25 %, 256x192 up to 2 x), where the reduction kernel's 256 CUs read the partials together.
 bool tile_fused_pays(const GemmArgs& g, int variant, int ksplit)
 {
-    (void)g;
-    return variant == TILE_64x64 && ksplit <= 8;
+    if (variant == TILE_64x64)
+        return ksplit <= 8;
+    if (variant == TILE_128x128) {
+        const long tiles = (long)((g.m + 127) / 128) * ((g.n + 127) / 128);
+        return ksplit <= 3 && tiles * ksplit >= 64;
+    }
+    return false;
+}
+
+// whether a tile plan that splits K would add its splits inside the kernel
+bool tile_plan_fused(const GemmArgs& g, int variant, int ksplit, const Config& cfg)
+{
+    if (ksplit <= 1 || !cfg.fused_ok || cfg.fused_mode == 0 || tile_mailbox_bytes(g, variant, ksplit) > SPLIT_MAILBOX_BYTES)
+        return false;
+    return cfg.fused_mode == 1 || tile_fused_pays(g, variant, ksplit);
 }
 
 // Shapes whose best measured plan differs from the model's choice: {m, n, k, variant, ksplit}.
@@ -229,15 +243,7 @@ void decide_persistent(const GemmArgs& g, Plan& p, const Config& cfg)
 // a tile to finish) or leaves them to the reduction kernel.
 void decide_fused(const GemmArgs& g, Plan& p, const Config& cfg)
 {
-    p.fused = false;
-    if (p.ksplit <= 1 || !cfg.fused_ok || cfg.fused_mode == 0)
-        return;
-    int bm, bn;
-    tile_variant_dims(p.variant, &bm, &bn);
-    const long tiles = (long)((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
-    if (tiles > TILE_TICKET_WORDS || (unsigned long long)g.m * g.n * 4ull * p.ksplit > 0x7FFFFFFFull)
-        return;
-    p.fused = cfg.fused_mode == 1 || tile_fused_pays(g, p.variant, p.ksplit);
+    p.fused = tile_plan_fused(g, p.variant, p.ksplit, cfg);
 }
 
 Plan make_plan(const GemmArgs& g, const Config& cfg)
@@ -380,7 +386,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             // for M = 16 ... 64: the best split never leaves a workgroup fewer than 8 K blocks)
             if (g.m <= 64 && fk <= 0 && selected == FP8GEMM_KERNEL_AUTO && ks > 1 && kbs < 8)
                 continue;
-            const double cst = tile_cost(g, v, ks);
+            const double cst = tile_cost(g, v, ks, tile_plan_fused(g, v, ks, cfg));
             if (cst < best) {
                 best = cst;
                 p.family = ks > 1 ? FP8GEMM_KERNEL_SPLITK : FP8GEMM_KERNEL_LARGE;
@@ -478,12 +484,13 @@ int acquire_workspace(size_t bytes, hipStream_t stream, Workspace* out)
 // bytes of partial sums a plan keeps behind the workspace header
 size_t plan_workspace_bytes(const GemmArgs& g, const Plan& p)
 {
-    if (p.ksplit <= 1 || (p.family == FP8GEMM_KERNEL_SKINNY && p.wide))  // the decode kernel's splits meet in the header
+    // splits that are added inside the kernel meet in the header
+    if (p.ksplit <= 1 || (p.family == FP8GEMM_KERNEL_SKINNY && p.wide) || p.fused)
         return 0;
     return (size_t)p.ksplit * g.m * g.n * sizeof(float);
 }
 // whether a plan uses the header although it keeps nothing behind it
-inline bool plan_uses_header(const Plan& p) { return p.family == FP8GEMM_KERNEL_SKINNY && p.wide && p.ksplit > 1; }
+inline bool plan_uses_header(const Plan& p) { return p.ksplit > 1 && ((p.family == FP8GEMM_KERNEL_SKINNY && p.wide) || p.fused); }
 // a workspace that holds `data` bytes of a plan: nothing, or the header and the data
 inline size_t with_header(size_t data, bool header_alone = false) { return data || header_alone ? data + WS_HEADER : 0; }
 
@@ -503,7 +510,6 @@ void plan_name(const Plan& p, char* out, size_t cap)
 // workspace whose zeroed header the plans use that add their K splits inside the kernel
 hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, const Workspace& w, hipStream_t stream)
 {
-    unsigned int* const tickets = ws_tickets(w);
     switch (p.family) {
     case FP8GEMM_KERNEL_SCALAR:
         return launch_scalar(g, stream);
@@ -514,7 +520,7 @@ hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, const W
     default: {
         if (p.persistent)
             return launch_tile_persistent(g, p.variant, NUM_CU, stream);
-        hipError_t e = launch_tile(g, p.variant, p.ksplit, partial, p.fused ? tickets : nullptr, stream);
+        hipError_t e = launch_tile(g, p.variant, p.ksplit, partial, p.fused ? ws_mailbox(w) : nullptr, stream);
         if (e == hipSuccess && p.ksplit > 1 && !p.fused)
             e = launch_splitk_reduce(g, p.ksplit, partial, stream);
         return e;
@@ -773,7 +779,7 @@ int run_grouped_table(const GroupTable& tab, int n, int k, bool decode, hipStrea
         const int nkb_i = k / 128;
         while (ksplit > 1 && (ksplit > nkb_i || (ksplit - 1) * ((nkb_i + ksplit - 1) / ksplit) >= nkb_i))
             --ksplit;
-        if (decode_grouped_mailbox_bytes(pt, n16, ksplit) > DECODE_MAILBOX_BYTES)
+        if (decode_grouped_mailbox_bytes(pt, n16, ksplit) > SPLIT_MAILBOX_BYTES)
             ksplit = 1;
     }
     Workspace w;
@@ -842,32 +848,42 @@ Config config_from_options(const fp8gemm_options* opt, int* rc)
 
 // aligned = the plan for 16-byte aligned operands; otherwise the larger of that and what the padded
 // plan needs when every operand has to be copied
-size_t workspace_bytes_for(int m, int n, int k, const Config& cfg, bool any_alignment)
+size_t workspace_bytes_for(int m, int n, int k, const Config& cfg_in, bool any_alignment)
 {
     if (m <= 0 || n <= 0 || k <= 0 || (k % 128) != 0)
         return 0;
     const uintptr_t al = 4096;
     GemmArgs g{reinterpret_cast<const uint8_t*>(al), reinterpret_cast<const uint8_t*>(al),
                reinterpret_cast<const float*>(al), nullptr, reinterpret_cast<uint16_t*>(al), m, n, k};
-    const Plan p = make_plan(g, cfg);
     GemmArgs gp = g;
     gp.m = (m + 15) & ~15;
     gp.n = (n + 15) & ~15;
     size_t need = 0;
-    if (p.family >= 0)
-        need = with_header(p.padded ? pad_layout(g, plan_workspace_bytes(gp, p), true, false).total
-                                    : plan_workspace_bytes(g, p), plan_uses_header(p));
-    if (any_alignment && !(p.family >= 0 && p.padded)) {
-        // the same shape with an operand off a 16-byte boundary: the plan of the padded shape on copies
-        const long long lim = 0x7FFFFFFFll;
-        if ((long long)gp.m * k <= lim && (long long)gp.n * k <= lim && (long long)gp.m * gp.n <= lim &&
-            cfg.selected != FP8GEMM_KERNEL_SCALAR) {
-            const Plan pp = make_plan(gp, cfg);
-            if (pp.family >= 0 && pp.family != FP8GEMM_KERNEL_SCALAR) {
-                const size_t all = with_header(pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total, plan_uses_header(pp));
-                need = all > need ? all : need;
+    // the larger need of the plans a call may settle on: with the K splits added inside the kernel, and
+    // -- when the device turns out not to place workgroups as that needs -- with the reduction kernel
+    for (int fused = 0; fused < 2; ++fused) {
+        Config cfg = cfg_in;
+        if (!fused)
+            cfg.fused_ok = false;
+        const Plan p = make_plan(g, cfg);
+        size_t one = 0;
+        if (p.family >= 0)
+            one = with_header(p.padded ? pad_layout(g, plan_workspace_bytes(gp, p), true, false).total
+                                       : plan_workspace_bytes(g, p), plan_uses_header(p));
+        if (any_alignment && !(p.family >= 0 && p.padded)) {
+            // the same shape with an operand off a 16-byte boundary: the plan of the padded shape on copies
+            const long long lim = 0x7FFFFFFFll;
+            if ((long long)gp.m * k <= lim && (long long)gp.n * k <= lim && (long long)gp.m * gp.n <= lim &&
+                cfg.selected != FP8GEMM_KERNEL_SCALAR) {
+                const Plan pp = make_plan(gp, cfg);
+                if (pp.family >= 0 && pp.family != FP8GEMM_KERNEL_SCALAR) {
+                    const size_t all = with_header(pad_layout(g, plan_workspace_bytes(gp, pp), true, false).total,
+                                                   plan_uses_header(pp));
+                    one = all > one ? all : one;
+                }
             }
         }
+        need = one > need ? one : need;
     }
     return need;
 }

@@ -377,7 +377,7 @@ bool decode_strip_supports(const GemmArgs& g)
 }
 
 // the mailbox of a K split: one patch per strip, sending split, wave and row tile
-bool decode_strip_can_split(const GemmArgs& g, int ksplit) { return decode_strip_mailbox_bytes(g, ksplit) <= DECODE_MAILBOX_BYTES; }
+bool decode_strip_can_split(const GemmArgs& g, int ksplit) { return decode_strip_mailbox_bytes(g, ksplit) <= SPLIT_MAILBOX_BYTES; }
 
 size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit)
 {
@@ -495,7 +495,7 @@ int decode_grouped_ksplit(const GroupTable& tab, int n, int k, bool fused_ok)
     int best = 1;
     double best_cost = decode_strip_cost(all, 1);
     for (int ks = 2; ks <= DECODE_MAX_KSPLIT && ks <= nkb; ++ks) {
-        if ((ks - 1) * ((nkb + ks - 1) / ks) >= nkb || decode_grouped_mailbox_bytes(tab, n, ks) > DECODE_MAILBOX_BYTES)
+        if ((ks - 1) * ((nkb + ks - 1) / ks) >= nkb || decode_grouped_mailbox_bytes(tab, n, ks) > SPLIT_MAILBOX_BYTES)
             continue;
         const double cst = decode_strip_cost(all, ks);
         if (cst < best_cost) {
@@ -513,7 +513,7 @@ hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit
     const long units = (long)strips * tab.groups;
     if (!decode_grouped_supports(tab, n, k) || ksplit < 1 || ksplit > nkb || ksplit > DECODE_MAX_KSPLIT ||
         units > 0x0FFFFFFF / DECODE_MAX_KSPLIT ||
-        (ksplit > 1 && (!mailbox || decode_grouped_mailbox_bytes(tab, n, ksplit) > DECODE_MAILBOX_BYTES)))
+        (ksplit > 1 && (!mailbox || decode_grouped_mailbox_bytes(tab, n, ksplit) > SPLIT_MAILBOX_BYTES)))
         return hipErrorInvalidValue;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     if ((ksplit - 1) * kb_per_split >= nkb)

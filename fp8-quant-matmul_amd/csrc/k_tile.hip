@@ -42,7 +42,7 @@ template <int BM, int BN, int WM, int WN, int NS, bool SPLIT>
 __global__ void __launch_bounds__(NTHREADS)
 tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                  const float* __restrict__ a_scale, const float* __restrict__ b_scale,
-                 uint16_t* __restrict__ c, float* __restrict__ partial, unsigned int* __restrict__ tickets,
+                 uint16_t* __restrict__ c, float* __restrict__ partial, float* mailbox,
                  int M, int lda, int N, int K, int tiles_m, int tiles_n, int kb_per_split, int group_m)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
@@ -292,112 +292,171 @@ tile_gemm_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
     for (; kb < kb1; ++kb)
         k_block(std::false_type{}, kb);
 
+    // ---- K splits added inside the kernel (mailbox != nullptr).  grid.x is a multiple of 8, so the
+    // workgroups of one tile (same blockIdx.x) have linear ids that agree modulo 8 and share an XCD: what
+    // they store and load meets in that XCD's L2.  The mailbox holds zeros between launches.  A wave of every
+    // split but the last stores its accumulators there in register order (1 KiB per instruction) with
+    // every +0.0 replaced by -0.0, so that no word it writes is zero, and is done.  The waves of the last
+    // split -- the workgroup with the highest id of its tile, dispatched after the others -- load the other
+    // splits' patches past their L1 until no word is zero, store zeros back, add them in split order, their
+    // own registers last (the arithmetic of splitk_reduce_kernel: adding -0.0 changes nothing), and the
+    // workgroup leaves through the bf16 epilogue.  A wave that has polled for a second gives up and
+    // writes NaN.
+    bool as_partial = SPLIT;
+    if constexpr (SPLIT) {
+        if (mailbox != nullptr) {
+            as_partial = false;
+            constexpr int PATCHES = NCW * MI * NJ;  // 32x32 patches of a tile: 4 KiB of fp32 each
+            const int senders = (int)gridDim.y - 1;
+            const size_t first = ((size_t)pid * senders * PATCHES + (size_t)wave * (MI * NJ)) * 256;  // in 16-byte units
+            if ((int)blockIdx.y < senders) {
+                if (compute) {
+                    v4i* mine = reinterpret_cast<v4i*>(mailbox) + first + (size_t)blockIdx.y * PATCHES * 256 + lane;
+#pragma unroll
+                    for (int i = 0; i < MI; ++i)
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                v4i bits;
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const int w = (int)__float_as_uint(acc[i][j][4 * q + e]);
+                                    bits[e] = w == 0 ? (int)0x80000000 : w;
+                                }
+                                mine[((i * NJ + j) * 4 + q) * 64] = bits;
+                            }
+                }
+                return;
+            }
+            if (compute) {
+                constexpr int ZC = MI * NJ <= 2 ? 4 : 2;  // splits polled together (registers)
+                const uint32_t span = (uint32_t)senders * PATCHES * 4096u;
+                const __amdgpu_buffer_rsrc_t rp = make_rsrc(reinterpret_cast<const v4i*>(mailbox) + first, span);
+                const unsigned long long t_first = __builtin_amdgcn_s_memrealtime();
+                bool gave_up = false;
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        v4f sum[4];
+                        for (int z0 = 0; z0 < senders; z0 += ZC) {
+                            v4i v[ZC][4];
+                            for (;;) {
+                                asm volatile("" ::: "memory");  // the loads belong to this round of the loop
+#pragma unroll
+                                for (int z = 0; z < ZC; ++z)
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q)  // a split past the last: outside the resource, zeros
+                                        v[z][q] = __builtin_amdgcn_raw_buffer_load_b128(
+                                            rp, (uint32_t)((((z0 + z) * PATCHES + i * NJ + j) * 4 + q) * 64 + lane) * 16u, 0, 16);
+                                bool missing = false;
+#pragma unroll
+                                for (int z = 0; z < ZC; ++z)
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q)
+                                        if (z0 + z < senders)
+                                            missing = missing || v[z][q][0] == 0 || v[z][q][1] == 0 || v[z][q][2] == 0 ||
+                                                      v[z][q][3] == 0;
+                                if (__builtin_amdgcn_ballot_w64(missing) == 0)
+                                    break;
+                                if (__builtin_amdgcn_s_memrealtime() - t_first > 100000000ull) {  // one second at 100 MHz
+                                    gave_up = true;
+                                    break;
+                                }
+                            }
+#pragma unroll
+                            for (int z = 0; z < ZC; ++z)
+                                if (z0 + z < senders) {
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q) {
+                                        __builtin_amdgcn_raw_buffer_store_b128(
+                                            (v4i){0, 0, 0, 0}, rp,
+                                            (uint32_t)((((z0 + z) * PATCHES + i * NJ + j) * 4 + q) * 64 + lane) * 16u, 0, 0);
+                                        const v4f f = __builtin_bit_cast(v4f, v[z][q]);
+                                        sum[q] = z0 + z == 0 ? f : sum[q] + f;
+                                    }
+                                }
+                        }
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                acc[i][j][4 * q + e] = gave_up ? __builtin_nanf("") : sum[q][e] + acc[i][j][4 * q + e];
+                    }
+            }
+        }
+    }
+
     // ---- epilogue.  A lane owns row m = .. + (lane & 31) and, per patch, four runs of 4 columns
     // (accumulator register 4*q + e is column 8*q + 4*(lane >> 5) + e of the patch): stored
     // straight from the registers that would be 8- or 16-byte pieces of 32 different rows per
     // instruction.  The tile therefore goes through the (now idle) LDS ring, row-major with a
     // padded row stride that keeps the writes conflict free, and leaves as 16 bytes per lane
     // along whole rows of the tile.  A tile larger than the ring is written in two halves.
-    constexpr int ESZ = SPLIT ? 4 : 2;
-    constexpr int CROW = BN * ESZ + (SPLIT ? 16 : 8);  // LDS bytes per tile row
-    constexpr int HALVES = (BM * CROW <= S::LDS_BYTES) ? 1 : 2;
-    constexpr int HROWS = BM / HALVES;
-    static_assert(HROWS * CROW <= S::LDS_BYTES, "half a tile must fit the ring");
-    static_assert(HROWS % 32 == 0, "a 32-row patch lies in one half");
-    constexpr int CPR = BN * ESZ / 16;                 // 16-byte chunks per tile row
-    constexpr int CHUNKS = HROWS * CPR;
+    // PARTIAL = fp32 into this split's partial tile (the reduction kernel follows), else bf16 into c.
+    auto write_tile = [&](auto partial_tag) __attribute__((always_inline)) {
+        constexpr bool PARTIAL = decltype(partial_tag)::value;
+        constexpr int ESZ = PARTIAL ? 4 : 2;
+        constexpr int CROW = BN * ESZ + (PARTIAL ? 16 : 8);  // LDS bytes per tile row
+        constexpr int HALVES = (BM * CROW <= S::LDS_BYTES) ? 1 : 2;
+        constexpr int HROWS = BM / HALVES;
+        static_assert(HROWS * CROW <= S::LDS_BYTES, "half a tile must fit the ring");
+        static_assert(HROWS % 32 == 0, "a 32-row patch lies in one half");
+        constexpr int CPR = BN * ESZ / 16;                 // 16-byte chunks per tile row
+        constexpr int CHUNKS = HROWS * CPR;
 #pragma unroll
-    for (int h = 0; h < HALVES; ++h) {
-        __syncthreads();  // nobody reads the ring (or the previous half) any more
+        for (int h = 0; h < HALVES; ++h) {
+            __syncthreads();  // nobody reads the ring (or the previous half) any more
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            const int prow = wm * TM + 32 * i;  // first tile row of the patch
-            if (compute && prow / HROWS == h) {
-                const uint32_t rbase = (uint32_t)((prow - h * HROWS + (lane & 31)) * CROW);
+            for (int i = 0; i < MI; ++i) {
+                const int prow = wm * TM + 32 * i;  // first tile row of the patch
+                if (compute && prow / HROWS == h) {
+                    const uint32_t rbase = (uint32_t)((prow - h * HROWS + (lane & 31)) * CROW);
 #pragma unroll
-                for (int j = 0; j < NJ; ++j)
+                    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int col = wn * TN + 32 * j + 8 * q + 4 * (lane >> 5);
-                        const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                       acc[i][j][4 * q + 3]};
-                        if (SPLIT) {
-                            *LDS_PTR(v4f, lds + rbase + col * 4) = v;
-                        } else {
-                            v2i pk = {(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3])};
-                            *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
+                        for (int q = 0; q < 4; ++q) {
+                            const int col = wn * TN + 32 * j + 8 * q + 4 * (lane >> 5);
+                            const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                           acc[i][j][4 * q + 3]};
+                            if (PARTIAL) {
+                                *LDS_PTR(v4f, lds + rbase + col * 4) = v;
+                            } else {
+                                v2i pk = {(int)pack_bf16x2(v[0], v[1]), (int)pack_bf16x2(v[2], v[3])};
+                                *LDS_PTR(v2i, lds + rbase + col * 2) = pk;
+                            }
                         }
-                    }
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int it = 0; it < (CHUNKS + NTHREADS - 1) / NTHREADS; ++it) {
-            const int idx = it * NTHREADS + (int)threadIdx.x;
-            const int row = idx / CPR, ch = idx - row * CPR;
-            const int mrow = m0 + h * HROWS + row;
-            const int ncol = n0 + ch * (16 / ESZ);
-            if (idx < CHUNKS && mrow < M && ncol < N) {
-                const size_t o = (size_t)mrow * N + ncol;
-                if (SPLIT) {
-                    const v4f v = *LDS_PTR(v4f, lds + row * CROW + ch * 16);
-                    *reinterpret_cast<v4f*>(partial + (size_t)blockIdx.y * M * N + o) = v;
-                } else {
-                    const v2i lo = *LDS_PTR(v2i, lds + row * CROW + ch * 16);
-                    const v2i hi = *LDS_PTR(v2i, lds + row * CROW + ch * 16 + 8);
-                    *reinterpret_cast<v4i*>(c + o) = (v4i){lo.x, lo.y, hi.x, hi.y};
                 }
             }
-        }
-    }
-
-    // ---- K splits added inside the kernel (tickets != nullptr).  grid.x is a multiple of 8, so the
-    // workgroups of one tile (same blockIdx.x) have linear ids that agree modulo 8 and share an XCD:
-    // the partial tiles meet in that XCD's L2.  Every thread waits for the L2's acknowledgement of its
-    // stores, the workgroup takes a ticket for the tile (workgroup-scope atomic, executed by that L2; it
-    // wraps to zero with the last arrival), and the workgroup that arrived last adds the partial tiles
-    // in split order -- the arithmetic of splitk_reduce_kernel, whoever arrives last -- and stores bf16.
-    if constexpr (SPLIT) {
-        if (tickets != nullptr) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();  // every thread's partial is in L2; nobody reads the staging area any more
-            auto flag = LDS_PTR(unsigned int, smem);
-            if (threadIdx.x == 0)
-                *flag = __builtin_amdgcn_atomic_inc32(tickets + pid, gridDim.y - 1, __ATOMIC_RELAXED, "workgroup");
             __syncthreads();
-            if (*flag != gridDim.y - 1)
-                return;
-            constexpr int QPR = BN / 4;                    // 16-byte pieces (4 floats) per tile row
-            constexpr int PIECES = BM * QPR / NTHREADS;    // per thread
-            static_assert(BM * QPR % NTHREADS == 0, "whole pieces per thread");
-            const size_t mn = (size_t)M * N;
-            const __amdgpu_buffer_rsrc_t rp = make_rsrc(partial, (uint32_t)(mn * 4u * gridDim.y));
-            v4f sum[PIECES];
-            uint32_t off[PIECES];
 #pragma unroll
-            for (int it = 0; it < PIECES; ++it) {
+            for (int it = 0; it < (CHUNKS + NTHREADS - 1) / NTHREADS; ++it) {
                 const int idx = it * NTHREADS + (int)threadIdx.x;
-                const int mrow = m0 + idx / QPR, ncol = n0 + (idx % QPR) * 4;
-                off[it] = (mrow < M && ncol < N) ? (uint32_t)(((size_t)mrow * N + ncol) * 4u) : 0x80000000u;
-            }
-            for (int z = 0; z < (int)gridDim.y; ++z) {
-                const uint32_t zoff = (uint32_t)(mn * 4u) * (uint32_t)z;
-#pragma unroll
-                for (int it = 0; it < PIECES; ++it) {  // loads past the L1 (sc1): served by the L2
-                    const v4f p = __builtin_bit_cast(
-                        v4f, __builtin_amdgcn_raw_buffer_load_b128(rp, off[it], zoff, 16));
-                    sum[it] = z == 0 ? p : sum[it] + p;
+                const int row = idx / CPR, ch = idx - row * CPR;
+                const int mrow = m0 + h * HROWS + row;
+                const int ncol = n0 + ch * (16 / ESZ);
+                if (idx < CHUNKS && mrow < M && ncol < N) {
+                    const size_t o = (size_t)mrow * N + ncol;
+                    if (PARTIAL) {
+                        const v4f v = *LDS_PTR(v4f, lds + row * CROW + ch * 16);
+                        *reinterpret_cast<v4f*>(partial + (size_t)blockIdx.y * M * N + o) = v;
+                    } else {
+                        const v2i lo = *LDS_PTR(v2i, lds + row * CROW + ch * 16);
+                        const v2i hi = *LDS_PTR(v2i, lds + row * CROW + ch * 16 + 8);
+                        *reinterpret_cast<v4i*>(c + o) = (v4i){lo.x, lo.y, hi.x, hi.y};
+                    }
                 }
             }
-#pragma unroll
-            for (int it = 0; it < PIECES; ++it)
-                if (off[it] != 0x80000000u) {
-                    uint2 pk;
-                    pk.x = pack_bf16x2(sum[it][0], sum[it][1]);
-                    pk.y = pack_bf16x2(sum[it][2], sum[it][3]);
-                    *reinterpret_cast<uint2*>(c + (off[it] >> 2)) = pk;
-                }
         }
+    };
+    if constexpr (SPLIT) {
+        if (as_partial)
+            write_tile(std::true_type{});
+        else
+            write_tile(std::false_type{});
+    } else {
+        write_tile(std::false_type{});
     }
 }
 
@@ -472,7 +531,7 @@ int choose_group_m(int tiles_m, int tiles_n, int bm, int bn)
 }
 
 template <int BM, int BN, int WM, int WN, int NS>
-hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, unsigned int* tickets, hipStream_t s)
+hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, float* mailbox, hipStream_t s)
 {
     using S = TileShape<BM, BN, WM, WN, NS>;
     constexpr int LDS_TOTAL = S::LDS_BYTES;
@@ -482,19 +541,19 @@ hipError_t launch_variant(const GemmArgs& g, int ksplit, float* partial, unsigne
     const int tiles = tiles_m * tiles_n;
     const int group_m = choose_group_m(tiles_m, tiles_n, BM, BN);
     if (ksplit > 1) {
-        // in-kernel reduction: one ticket per tile, partial tiles addressed with 32-bit offsets
-        if (tickets && (tiles > TILE_TICKET_WORDS || (unsigned long long)g.m * g.n * 4ull * ksplit > 0x7FFFFFFFull))
+        // in-kernel reduction: the other splits' patches of every tile fit the mailbox
+        if (mailbox && (size_t)tiles * (ksplit - 1) * BM * BN * 4 > SPLIT_MAILBOX_BYTES)
             return hipErrorInvalidValue;
-        dim3 grid(tickets ? (tiles + 7) & ~7 : tiles, ksplit);
+        dim3 grid(mailbox ? (tiles + 7) & ~7 : tiles, ksplit);
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, true>;
         FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
         hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale, g.c, partial,
-                           tickets, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
+                           mailbox, g.m, leading_dim(g), g.n, g.k, tiles_m, tiles_n, kb_per_split, group_m);
     } else {
         auto kern = tile_gemm_kernel<BM, BN, WM, WN, NS, false>;
         FP8GEMM_ALLOW_LDS(kern, LDS_TOTAL);
         hipLaunchKernelGGL(kern, dim3(tiles, 1), dim3(NTHREADS), LDS_TOTAL, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
-                           partial, static_cast<unsigned int*>(nullptr), g.m, leading_dim(g), g.n, g.k, tiles_m,
+                           partial, static_cast<float*>(nullptr), g.m, leading_dim(g), g.n, g.k, tiles_m,
                            tiles_n, kb_per_split, group_m);
     }
     return hipGetLastError();
@@ -540,15 +599,23 @@ void tile_variant_dims(int variant, int* bm, int* bn)
     }
 }
 
-hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, unsigned int* tickets,
+size_t tile_mailbox_bytes(const GemmArgs& g, int variant, int ksplit)
+{
+    int bm, bn;
+    tile_variant_dims(variant, &bm, &bn);
+    const size_t tiles = (size_t)((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
+    return ksplit > 1 ? tiles * (size_t)(ksplit - 1) * bm * bn * 4 : 0;
+}
+
+hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, float* mailbox,
                        hipStream_t s)
 {
     switch (variant) {
-    case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, tickets, s);
-    case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, tickets, s);
-    case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, tickets, s);
-    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, tickets, s);
-    case TILE_64x64: return launch_variant<64, 64, 2, 2, 4>(g, ksplit, partial, tickets, s);
+    case TILE_256x192: return launch_variant<256, 192, 4, 2, 2>(g, ksplit, partial, mailbox, s);
+    case TILE_256x128: return launch_variant<256, 128, 4, 2, 3>(g, ksplit, partial, mailbox, s);
+    case TILE_128x192: return launch_variant<128, 192, 4, 2, 3>(g, ksplit, partial, mailbox, s);
+    case TILE_128x128: return launch_variant<128, 128, 2, 4, 4>(g, ksplit, partial, mailbox, s);
+    case TILE_64x64: return launch_variant<64, 64, 2, 2, 4>(g, ksplit, partial, mailbox, s);
     default: return hipErrorInvalidValue;
     }
 }

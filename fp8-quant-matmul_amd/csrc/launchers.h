@@ -45,18 +45,23 @@ inline int leading_dim(const GemmArgs& g) { return g.lda ? g.lda : g.m; }
 // one thread per C element (check.cu:30-49)
 hipError_t launch_scalar(const GemmArgs& g, hipStream_t s);
 
+// The mailbox: device memory that only the kernels that add their K splits themselves write, all zero
+// before a launch and all zero again after it; the splits of a tile or strip hand their partial results
+// over through it.
+constexpr size_t SPLIT_MAILBOX_BYTES = (size_t)16 << 20;
+
 // MFMA tile kernel family.  `variant` picks the workgroup tile; ksplit > 1 writes fp32
-// partial sums to `partial` ([ksplit][m][n]) instead of c.  With tickets == nullptr it must be followed
-// by launch_splitk_reduce; with tickets (TILE_TICKET_WORDS words, zero before the launch and zero again
-// after it) the workgroup of a tile that finishes last adds the partial tiles itself and writes c, with
-// the same arithmetic.  The latter needs xcd_placement_confirmed() and at most TILE_TICKET_WORDS tiles.
+// partial sums to `partial` ([ksplit][m][n]) instead of c.  With mailbox == nullptr it must be followed
+// by launch_splitk_reduce; with a mailbox (SPLIT_MAILBOX_BYTES) the workgroup of a tile's last split
+// adds the other splits' accumulators itself and writes c, with the same arithmetic, and `partial` is
+// not used.  The latter needs xcd_placement_confirmed() and tile_mailbox_bytes() <= SPLIT_MAILBOX_BYTES.
 enum TileVariant { TILE_256x192 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_128x192 = 3,
                    TILE_64x64 = 4, TILE_256x192_W4 = 5, TILE_256x256 = 6, TILE_VARIANT_COUNT };
 bool tile_supports(const GemmArgs& g);
 const char* tile_variant_name(int variant);
 void tile_variant_dims(int variant, int* bm, int* bn);
-constexpr int TILE_TICKET_WORDS = 4096;
-hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, unsigned int* tickets,
+size_t tile_mailbox_bytes(const GemmArgs& g, int variant, int ksplit);
+hipError_t launch_tile(const GemmArgs& g, int variant, int ksplit, float* partial, float* mailbox,
                        hipStream_t s);
 // Persistent form (ksplit = 1 only): `workgroups` (a multiple of 8) workgroups walk through
 // all tiles, the copies of a tile's first K blocks overlap the previous tile's epilogue.
@@ -87,10 +92,8 @@ double skinny_cost(const GemmArgs& g, int ksplit);
 hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStream_t s);
 
 // wide-strip decode kernel (M <= 64): 128-column strips, the K splits of a strip added inside the
-// kernel.  `mailbox` = DECODE_MAILBOX_BYTES of device memory that only this kernel writes, all zero before
-// the launch and all zero again after it (the splits hand their partial patches over through it).
-// ksplit > 1 needs xcd_placement_confirmed() and decode_strip_can_split.
-constexpr size_t DECODE_MAILBOX_BYTES = (size_t)8 << 20;
+// kernel.  `mailbox` = SPLIT_MAILBOX_BYTES as above.  ksplit > 1 needs xcd_placement_confirmed() and
+// decode_strip_can_split.
 constexpr int DECODE_MAX_KSPLIT = 16;
 bool decode_strip_supports(const GemmArgs& g);
 size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit);

@@ -108,10 +108,11 @@ int fp8_block_gemm_set_persistent(int mode);
 
 /* Plans that split K ("..._kN") write fp32 partial results; they are added either by a second kernel or
  * inside the GEMM kernel ("..._kNf", "decode128_kN"): the K splits of a tile are placed on one XCD and meet
- * in its L2.  Tile kernels count themselves in with a ticket and the workgroup that finishes a tile last adds
- * the partials in split order, so the result does not depend on who is last and equals the second kernel's
- * bit for bit; in the decode kernel the waves of the last split poll a zero-initialised mailbox for the other
- * splits' partial patches and add them in split order (a wave that polls for a second writes NaN).  mode -1 = by cost (default), 0 = never,
+ * in its L2.  Every split but the last stores its accumulators into a zero-initialised mailbox (with +0.0
+ * written as -0.0, so that no word is zero); the waves of the last split poll the mailbox until nothing is
+ * missing, store zeros back and add the partials in split order, their own last -- the second kernel's
+ * arithmetic, so the result equals its bit for bit and does not depend on timing (a wave that polls for a
+ * second gives up and writes NaN).  mode -1 = by cost (default), 0 = never,
  * 1 = whenever the plan allows.  The first call that could use it on a device looks once at where that
  * device places workgroups (a probe grid the call waits for; skipped, and the two-kernel form used, while
  * the stream is being captured and the answer is not known yet).  The reference does not split K
@@ -157,12 +158,12 @@ typedef struct fp8gemm_options {
 /* The first FP8GEMM_WORKSPACE_HEADER_BYTES of the workspace handed to this call were zero-filled by the
  * caller before the first call that used this workspace, and nothing but this library has written to the
  * workspace since.  The plans that add the K splits of a tile or strip inside the GEMM kernel instead of
- * launching a reduction kernel ("decode128_kN", "..._kNf") keep their hand-over state there -- arrival
- * tickets (16 KiB) and the decode kernel's mailbox of partial patches (8 MiB) -- and leave all of it zero
- * again after every call; without the flag a per-call workspace only gets the two-kernel plans.
+ * launching a reduction kernel ("decode128_kN", "..._kNf") hand their partial results over through it (a
+ * mailbox of 16 MiB) and leave all of it zero again after every call; without the flag a per-call workspace
+ * only gets the two-kernel plans.
  * The process-wide workspace and fp8_block_gemm_noalloc's array always have a zeroed header. */
 #define FP8GEMM_FLAG_WORKSPACE_ZEROED 1
-#define FP8GEMM_WORKSPACE_HEADER_BYTES (16384 + (8u << 20))
+#define FP8GEMM_WORKSPACE_HEADER_BYTES (16u << 20)
 int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
                       int m, int n, int k, const fp8gemm_options* options, void* workspace,
                       size_t workspace_bytes, void* stream);

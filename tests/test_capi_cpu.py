@@ -216,7 +216,7 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(8191, 4607, 7168) == "padded_" + pkg.plan(8192, 4608, 7168)
     assert pkg.plan(16777215, 16, 128) == "scalar"         # padding would pass the operand size limit
     assert pkg.workspace_bytes(33, 100, 128) >= 128 * 48 + 128 * 112 + 48 * 4 + 48 * 112 * 2
-    ks = int(pkg.plan(2048, 576, 7168).split("_k")[1])
+    ks = int(pkg.plan(2048, 576, 7168).split("_k")[1].rstrip("f"))
     assert ks > 1                                          # few tiles, long K: split
     # decode shapes (M <= 32): 128-column strips with the K range split so that one round of workgroups
     # (at most 256) streams B, the splits added inside the kernel
@@ -240,11 +240,21 @@ def test_dispatcher_plans(pkg):
     pkg.set_fused_reduction(0)                             # reduction kernel instead of the in-kernel reduction
     try:
         assert pkg.plan(64, 1536, 7168) == "tile64x64_k7" and pkg.plan(32, 7168, 2048) == "skinny_k1"
+        assert pkg.plan(2048, 576, 7168) == "tile128x128_k3"
         pkg.set_fused_reduction(1)
-        assert pkg.plan(2048, 576, 7168).endswith("f")
+        pkg.select(pkg.KERNEL_SPLITK)
+        pkg.force_config(1, 3)
+        assert pkg.plan(2048, 576, 7168) == "tile256x128_k3f"   # whenever the other splits' tiles fit the mailbox
+        pkg.force_config(1, 6)
+        assert pkg.plan(2048, 576, 7168) == "tile256x128_k6"    # 40 tiles x 5 x 128 KiB do not
+        pkg.force_config(-1, 0)
+        pkg.select(pkg.KERNEL_AUTO)
     finally:
         pkg.set_fused_reduction(-1)
-    assert not pkg.plan(2048, 576, 7168).endswith("f")     # 128x128 tiles: the reduction kernel is faster
+        pkg.force_config(-1, 0)
+        pkg.select(pkg.KERNEL_AUTO)
+    assert pkg.plan(2048, 576, 7168) == "tile128x128_k3f"   # two or three splits of 128x128 tiles: inside the kernel
+    assert pkg.plan(512, 512, 4096).startswith("tile64x64_k") and pkg.plan(512, 512, 4096).endswith("f")
     pkg.select(pkg.KERNEL_SCALAR)
     assert pkg.plan(8192, 4608, 7168) == "scalar"
     pkg.select(pkg.KERNEL_SKINNY)

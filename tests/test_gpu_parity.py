@@ -195,7 +195,7 @@ def test_tile_kernel_256x256(pkg, m, n, k):
                                                    (1, 3, 272, 576, 896), (0, 8, 256, 576, 2048),
                                                    (2, 7, 128, 640, 7168), (1, 16, 256, 128, 2048), (3, 5, 384, 576, 1280),
                                                    (4, 3, 208, 336, 768), (4, 2, 64, 64, 256),
-                                                   (2, 3, 2048, 576, 1536), (4, 4, 1008, 528, 1024), (4, 16, 512, 512, 2048)])
+                                                   (2, 3, 2048, 576, 1536), (4, 4, 1008, 528, 1024), (4, 8, 512, 512, 2048)])
 def test_tile_kernel_split_k(pkg, variant, ksplit, m, n, k):
     """the K range split over workgroups: partial tiles added by the reduction kernel (fused=0) and by the
     last workgroup of each tile inside the GEMM kernel (fused=1) -- same sums in the same order"""
@@ -258,11 +258,11 @@ def test_decode_strip_kernel(pkg, m, n, k, ksplit):
 
 
 def test_decode_strip_split_that_outgrows_the_mailbox_is_refused(pkg):
-    """128 strips x 7 sending splits x 16 KiB of patches do not fit the 8 MiB mailbox: no such plan"""
-    m, n, k = 32, 16384, 1024
+    """128 strips x 15 sending splits x 16 KiB of patches do not fit the 16 MiB mailbox: no such plan"""
+    m, n, k = 32, 16384, 2048
     a, b, sa, sb = oracle.make_inputs(m, n, k, 1290)
     with pytest.raises(pkg.Fp8GemmError) as info:
-        _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=8)
+        _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=16)
     assert info.value.code == -3
 
 
