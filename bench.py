@@ -51,13 +51,13 @@ CHALLENGE_REF_GEOMEAN_US = 136.0
 # reads 0.5 of the bytes copied (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 # profiles/counters_cfg1_to_cfg5.md holds the table; the kernels measured are those of the commit
 # named here (the kernels of these plans have not changed since).
-TRAFFIC_MEASURED_AT_COMMIT = "03b9e4e"
+TRAFFIC_MEASURED_AT_COMMIT = "d3f0c1a"
 MEASURED_TRAFFIC_BYTES = {
-    "cfg1": int((4191 * 2.0 + 1024 * 1.0) * 1024),       # 9.6 MB
-    "cfg2": int((115834 * 2.0 + 114688 * 1.0) * 1024),   # 355 MB
-    "cfg3": int((30491 * 2.0 + 16128 * 1.0) * 1024),     # 79 MB, tile kernel + reduction
-    "cfg4": int((242080 * 2.0 + 73728 * 1.0) * 1024),    # 571 MB: 8 L2s refetch A/B panels
-    "cfg5": int((7462 * 2.0 + 448 * 1.0) * 1024),        # 15.7 MB: 1.04 x the algorithmic bytes
+    "cfg1": int((5235 * 2.0 + 3072 * 1.0) * 1024),       # 13.9 MB: C + the mailbox traffic of the K split
+    "cfg2": int((115831 * 2.0 + 114688 * 1.0) * 1024),   # 355 MB
+    "cfg3": int((28731 * 2.0 + 20315 * 1.0) * 1024),     # 79.6 MB, one kernel (K splits added inside it)
+    "cfg4": int((242077 * 2.0 + 73728 * 1.0) * 1024),    # 571 MB: 8 L2s refetch A/B panels
+    "cfg5": int((8841 * 2.0 + 3136 * 1.0) * 1024),       # 21.3 MB: B once (1.23 x the reads) + mailbox write-back
 }
 
 
@@ -416,6 +416,51 @@ def main():
                 out["kernel"] = pkg.last_kernel()
         return out
 
+    def grouped_decode_report(steps, warmup, experts=64, gn=7168, gk=2048, on_grid=False):
+        """an MoE layer in a decode step: `experts` problems of 1 to 64 rows each (seeded), every expert with
+        its own weights (64 x 14.7 MB: streamed from HBM on every launch).  One grouped call (one launch of
+        the decode kernel on all experts' strips) against one call per expert.  Operands are seeded random
+        bytes and scales generated on the device (parity of the grouped path is the tests' business)."""
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(4242)
+        rs = __import__("numpy").random.RandomState(4242)
+        ms = [int(v) for v in rs.randint(1, 65, size=experts)]
+        if on_grid:
+            ms = [max(16, (v + 15) // 16 * 16) for v in ms]
+        bufs = []
+        for gm in ms:
+            a_ = torch.randint(0, 120, (gk, gm), device="cuda", generator=gen, dtype=torch.int16).to(torch.uint8)
+            b_ = torch.randint(0, 120, (gk, gn), device="cuda", generator=gen, dtype=torch.int16).to(torch.uint8)
+            sa_ = torch.rand((gk // 128, gm), device="cuda", generator=gen) + 0.5
+            sb_ = torch.rand((gk // 128, (gn + 127) // 128), device="cuda", generator=gen) + 0.5
+            bufs.append([a_, b_, sa_, sb_, torch.zeros((gm, gn), dtype=torch.int16, device="cuda")])
+        cols = lambda i: [bf[i] for bf in bufs]
+        grouped = lambda: pkg.gemm_grouped(cols(0), cols(1), cols(2), cols(3), cols(4), ms, gn, gk, sptr)
+
+        def one_by_one():
+            for bf, gm in zip(bufs, ms):
+                pkg.gemm(bf[0], bf[1], bf[2], bf[3], bf[4], gm, gn, gk, sptr)
+
+        byts = sum(algorithmic_work(gm, gn, gk)[1] for gm in ms)
+        out = {"experts": experts, "rows_total": sum(ms), "rows_min_max": [min(ms), max(ms)], "n": gn, "k": gk,
+               "algorithmic_bytes": byts}
+        for tag, fn in (("grouped", grouped), ("one_by_one", one_by_one)):
+            settle(fn, warmup)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / steps
+            out[tag + "_us"] = round(us, 2)
+            out[tag + "_gbs"] = round(byts / us * 1e-3, 1)
+            out[tag + "_kernel"] = pkg.last_kernel()
+        out["grouped_frac_hbm_peak"] = round(out["grouped_gbs"] / PEAK_HBM_GBS, 4)
+        pkg.release()
+        return out
+
     def launch_floor_us(reps=200):
         """back-to-back launches of a one-workgroup kernel of this library"""
         x = torch.zeros(256, dtype=torch.float32, device="cuda")
@@ -455,6 +500,10 @@ def main():
     if grouped is not None:   # the same token count with group sizes off the 16-row grid: padded copies
         grouped["off_grid"] = grouped_report(max(30, args.steps), args.warmup,
                                              ms=(509, 1027, 771, 1533, 250, 2051, 1023, 1028))
+    grouped_decode = None
+    if not args.no_shapes:   # 64 experts of 1..64 rows (padded copies of A), and the same on the 16-row grid
+        grouped_decode = grouped_decode_report(max(20, args.steps), args.warmup)
+        grouped_decode["on_grid"] = grouped_decode_report(max(20, args.steps), args.warmup, on_grid=True)
     host_boundary = None if args.no_shapes else host_boundary_report()
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
@@ -516,6 +565,7 @@ def main():
         "quantisers": quantisers,
         "vendor_plain_fp8_gemm": vendor,
         "grouped": grouped,
+        "grouped_decode": grouped_decode,
         "host_boundary": host_boundary,
         "device": device,
     }

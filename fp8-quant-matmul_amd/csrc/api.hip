@@ -33,8 +33,8 @@ struct Config {
     int force_variant;  // tile shape, -1 = cost model
     int force_ksplit;   // 0 = cost model
     int persistent;     // -1 / 0 / 1 as above
-    // plans that add K splits inside the kernel may be chosen: the workspace starts with zeroed ticket
-    // words and the device places workgroups on XCDs as those kernels assume (set by run())
+    // plans that add K splits inside the kernel may be chosen: the workspace starts with a zeroed header
+    // and the device places workgroups on XCDs as those kernels assume (set by run())
     bool fused_ok = true;
     int fused_mode = -1;  // -1 = by cost, 0 = never, 1 = whenever fused_ok and the plan allows
 };
@@ -283,7 +283,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             narrow_us = skinny_cost(g, narrow.ksplit);
         }
         if (wide_ok && (by_name ? cfg.force_variant != 0 : cfg.force_variant < 0)) {
-            // without the in-kernel reduction (no zeroed tickets, or workgroup placement not confirmed) only
+            // without the in-kernel reduction (no zeroed mailbox, or workgroup placement not confirmed) only
             // the unsplit form exists
             const int hi = cfg.fused_ok ? (nkb < MAX_KSPLIT ? nkb : MAX_KSPLIT) : 1;
             for (int ks = 1; ks <= hi; ++ks) {
@@ -452,7 +452,7 @@ int acquire_workspace(size_t bytes, hipStream_t stream, Workspace* out)
         }
         if (e != hipSuccess)
             return (int)e;
-        e = hipMemset(p, 0, WS_HEADER);  // the ticket words (bytes >= WS_HEADER whenever a plan needs a workspace)
+        e = hipMemset(p, 0, WS_HEADER);  // the mailbox (bytes >= WS_HEADER whenever a plan needs a workspace)
         if (e != hipSuccess) {
             (void)hipFree(p);
             return (int)e;
@@ -603,7 +603,7 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
         return v;
     GemmArgs g{static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), as, bs,
                static_cast<uint16_t*>(c), m, n, k};
-    // in-kernel K-split reduction: zeroed ticket words (every process-wide workspace has them; a per-call
+    // in-kernel K-split reduction: a zeroed header (every process-wide workspace has one; a per-call
     // one when the caller says so) and a confirmed workgroup placement
     cfg.fused_ok = cfg.fused_ok && (!explicit_ws || explicit_ws->zeroed);
     if (cfg.fused_ok) {
@@ -1170,8 +1170,8 @@ int fp8_block_gemm_set_workspace(void* device_ptr, size_t bytes)
 {
     if (device_ptr && (reinterpret_cast<uintptr_t>(device_ptr) % 256) != 0)
         return FP8GEMM_E_WORKSPACE;
-    // the ticket words at its start are zero-filled here (the call waits for that fill); a buffer too
-    // small to hold them can serve no plan anyway
+    // the header at its start is zero-filled here (the call waits for that fill); a buffer too
+    // small to hold it can serve no plan anyway
     bool zeroed = false;
     if (device_ptr && bytes >= WS_HEADER) {
         const hipError_t e = hipMemset(device_ptr, 0, WS_HEADER);

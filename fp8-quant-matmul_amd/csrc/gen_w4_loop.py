@@ -123,23 +123,12 @@ def scale_wait(g):
 
 
 # ---- text
-# --ablate a,b,..: leave a class of instructions out to see what it costs (TIMING ONLY: the results
-# are wrong).  copy = global->LDS copies, barrier, read = fragment reads, fold = FMAs, wait = LDS waits,
-# nop = padding
-ABLATE = set()
-ABLATIONS = {"copy": ("buffer_load",), "barrier": ("s_barrier", "s_waitcnt vmcnt"), "read": ("ds_read_b64_tr_b8",),
-             "fold": ("v_fmac_f32",), "wait": ("s_waitcnt lgkmcnt",), "nop": ("s_nop",)}
-
-
 class Asm:
-    def __init__(self, ablate=True):
+    def __init__(self):
         self.lines = []
         self.skippable = set()   # indices of instructions a taken branch jumps over
-        self.ablate = ablate
 
     def __call__(self, text, skippable=False):
-        if self.ablate and any(text.startswith(pre) for name in ABLATE for pre in ABLATIONS[name]):
-            return
         if skippable:
             self.skippable.add(len(self.lines))
         self.lines.append(text)
@@ -361,7 +350,7 @@ def emit_loop(out):
 
 
 def emit_first_reads(out):
-    a = Asm(ablate=False)
+    a = Asm()
     for c in range(GAPS_COL):
         for op in gap_ops((NJ - 1) * GAPS_COL + c):
             if op[0] == "A":
@@ -388,7 +377,7 @@ def emit_first_reads(out):
 
 
 def emit_drain(out):
-    a = Asm(ablate=False)
+    a = Asm()
     a("s_nop 15")
     a(f"s_nop {MFMA_RESULT_SLOTS - 16 - 1}")
     fold_part(a, NP - 1, (NP - 1) & 1, 0, 16)
@@ -406,11 +395,7 @@ def emit_drain(out):
 
 
 def main():
-    if len(sys.argv) > 2 and sys.argv[1] == "--ablate":
-        ABLATE.update(sys.argv[2].split(","))
-        assert ABLATE <= set(ABLATIONS), f"unknown ablation in {ABLATE}"
-    out = ["// GENERATED by gen_w4_loop.py -- do not edit; schedule and register map are documented there."
-           + (f"  ABLATED (timing only, wrong results): {sorted(ABLATE)}" if ABLATE else ""),
+    out = ["// GENERATED by gen_w4_loop.py -- do not edit; schedule and register map are documented there.",
            f"// STAGE = {STAGE} bytes per ring slot; MFMA waits: " + " ".join(str(mfma_wait(g)) for g in range(NG)),
            ""]
     emit_loop(out)

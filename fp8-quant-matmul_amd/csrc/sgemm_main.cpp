@@ -1,7 +1,7 @@
 // Timing driver: the procedure of /root/reference/sgemm.cu:89-127 (10 launches bracketed by
 // events, first one dropped, mean of the remaining 9 in microseconds), on the full grid
 // (the reference's timed cases launch half of it, sgemm.cu:106).  Inputs are resident on the
-// device before the timed region.  Usage: sgemm M N K [runs [tile_variant [ksplit [constant [warmup]]]]]
+// device before the timed region.  Usage: sgemm M N K [runs [tile_variant [ksplit [constant [warmup [b_copies]]]]]]
 // (tile_variant / ksplit pin the kernel plan as fp8_block_gemm_force_config does, -1 / 0 leave
 // the choice to the dispatcher; constant = 1 fills both operands with the single code 0x38
 // instead of the seed-7 stream: same instructions, no toggling operand bits, i.e. the run
@@ -10,7 +10,9 @@
 // of A and per 128 x 128 block of B, codes with sign bits and full mantissas): the load the
 // headline figure is measured on; warmup = untimed launches issued back to
 // back right before the timed ones: after an idle gap the part needs ~30 ms of continuous load
-// to reach its steady clock, which the reference's ten-launch procedure never sees)
+// to reach its steady clock, which the reference's ten-launch procedure never sees; b_copies > 1 keeps that
+// many copies of B on the device and gives every launch, warm-up included, the next one in turn: with
+// more copies than the caches hold, B comes from HBM on every launch)
 #include "host_harness.h"
 
 #include <hip/hip_runtime.h>
@@ -59,12 +61,16 @@ int main(int argc, char** argv)
 
     void *da, *db, *das, *dbs, *dc;
     CHECK(hipMalloc(&da, a8.size()));
-    CHECK(hipMalloc(&db, b8.size()));
+    const int b_copies = argc > 9 && std::atoi(argv[9]) > 1 ? std::atoi(argv[9]) : 1;
+    CHECK(hipMalloc(&db, b8.size() * (size_t)b_copies));
     CHECK(hipMalloc(&das, as.size() * 4));
     CHECK(hipMalloc(&dbs, bs.size() * 4));
     CHECK(hipMalloc(&dc, M * N * 2));
     CHECK(hipMemcpy(da, a8.data(), a8.size(), hipMemcpyHostToDevice));
-    CHECK(hipMemcpy(db, b8.data(), b8.size(), hipMemcpyHostToDevice));
+    for (int i = 0; i < b_copies; ++i)
+        CHECK(hipMemcpy((uint8_t*)db + (size_t)i * b8.size(), b8.data(), b8.size(), hipMemcpyHostToDevice));
+    int turn = 0;
+    auto next_b = [&]() { return (const void*)((const uint8_t*)db + (size_t)(turn++ % b_copies) * b8.size()); };
     CHECK(hipMemcpy(das, as.data(), as.size() * 4, hipMemcpyHostToDevice));
     CHECK(hipMemcpy(dbs, bs.data(), bs.size() * 4, hipMemcpyHostToDevice));
 
@@ -75,13 +81,13 @@ int main(int argc, char** argv)
     CHECK(hipEventCreate(&stop));
     const int warmup = argc > 8 ? std::atoi(argv[8]) : 0;
     for (int i = 0; i < warmup; ++i)
-        if (fp8_block_gemm_stream(da, db, (const float*)das, (const float*)dbs, dc, (int)M, (int)N, (int)K,
+        if (fp8_block_gemm_stream(da, next_b(), (const float*)das, (const float*)dbs, dc, (int)M, (int)N, (int)K,
                                   stream) != 0)
             return 2;
     float total = 0.f;
     for (int i = 0; i < runs; ++i) {
         CHECK(hipEventRecord(start, stream));
-        int rc = fp8_block_gemm_stream(da, db, (const float*)das, (const float*)dbs, dc, (int)M, (int)N,
+        int rc = fp8_block_gemm_stream(da, next_b(), (const float*)das, (const float*)dbs, dc, (int)M, (int)N,
                                        (int)K, stream);
         if (rc != 0) {
             std::fprintf(stderr, "fp8_block_gemm: %s\n", fp8_block_gemm_error_string(rc));

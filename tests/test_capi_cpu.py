@@ -111,7 +111,7 @@ def test_workspace_contract(pkg):
     assert pkg.workspace_bytes(64, 64, 128) == 0                     # one K block: nothing to split
     assert pkg.workspace_bytes(8192, 4608, 7168) == 0                # plan does not split K
     assert pkg.plan(1024, 512, 7168) == "tile64x64_k2f"                # f: the K splits are added inside the kernel
-    H = pkg.WORKSPACE_HEADER_BYTES                                   # ticket words ahead of every plan's data
+    H = pkg.WORKSPACE_HEADER_BYTES                                   # the mailbox ahead of every plan's data
     assert pkg.workspace_bytes(1024, 512, 7168) == H + 2 * 1024 * 512 * 4
     assert L.fp8_block_gemm_force_config(2, 8) == 0                  # follows a forced configuration
     try:

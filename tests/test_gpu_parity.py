@@ -159,7 +159,7 @@ def test_tile_kernel_one_wave_per_simd(pkg, m, n, k):
     assert np.array_equal(got, again), "run-to-run reproducible"
 
 
-# the last three: more tiles x splits than CUs (several rounds of workgroups meet at the tickets), a tile
+# the last three: more tiles x splits than CUs (several rounds of workgroups meet in the mailbox), a tile
 # count that is not a multiple of 8 with ragged edges, many splits of many small tiles
 @pytest.mark.parametrize("m,n,k", [(250, 300, 512), (1000, 200, 256), (4000, 3000, 128), (272, 192, 128)])
 def test_tile_kernel_one_wave_per_simd_off_the_grid(pkg, m, n, k):
@@ -292,7 +292,7 @@ def test_decode_strip_mailbox_survives_a_change_of_shape(pkg):
 
 
 def test_decode_strips_in_a_caller_workspace_need_its_zeroed_flag(pkg):
-    """fp8_block_gemm_ex: the in-kernel reduction keeps its hand-over state (tickets, the decode kernel's
+    """fp8_block_gemm_ex: the in-kernel reduction keeps its hand-over state (the
     mailbox) in the header of the workspace, so a per-call workspace gets it only when the caller vouches for
     a zeroed header; without the flag the call takes a plan that needs none"""
     import torch

@@ -1,6 +1,6 @@
 """fp8_block_gemm_noalloc: the entry point whose workspace is a fixed array in the library's device
 image.  Called through the C ABI on plans that use that workspace (a K split, padded copies, the decode
-kernel's tickets and partial patches), twice in a row with the second problem smaller, against
+kernel's and the tile kernels' mailbox), twice in a row with the second problem smaller, against
 fp8_block_gemm_stream on the same inputs: bit for bit.  The calls must leave the device's free memory
 and the library-owned workspace untouched, and must work under stream capture, where the stream entry
 point is refused for want of a workspace."""
@@ -19,11 +19,11 @@ def _say(msg):
     sys.stdout.flush()
 
 
-CASES = [(2048, 576, 7168, 8501, "_k3"),      # K split: 14 MB of fp32 partials in the fixed array
+CASES = [(2048, 576, 7168, 8501, "_k3"),      # K split added inside the kernel: the mailbox at the start of the fixed array
          (1024, 512, 7168, 8502, "_k2"),      # a smaller problem right after, same array
          (250, 300, 512, 8503, "padded_"),    # padded copies
-         (32, 7168, 2048, 8505, "decode128_k4"),   # tickets and partial patches of the decode kernel
-         (16, 1536, 1024, 8506, "decode128_k"),    # fewer strips right after, same tickets
+         (32, 7168, 2048, 8505, "decode128_k4"),   # the decode kernel's splits meet in the same mailbox
+         (16, 1536, 1024, 8506, "decode128_k"),    # fewer strips right after, same mailbox
          (8192, 4608, 256, 8504, "_k1")]      # needs no workspace at all
 
 
