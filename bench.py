@@ -51,7 +51,7 @@ CHALLENGE_REF_GEOMEAN_US = 136.0
 # reads 0.5 of the bytes copied (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 # profiles/counters_cfg1_to_cfg5.md holds the table; the kernels measured are those of the commit
 # named here (the kernels of these plans have not changed since).
-TRAFFIC_MEASURED_AT_COMMIT = "d3f0c1a"
+TRAFFIC_MEASURED_AT_COMMIT = "a37a2c8"
 MEASURED_TRAFFIC_BYTES = {
     "cfg1": int((5235 * 2.0 + 3072 * 1.0) * 1024),       # 13.9 MB: C + the mailbox traffic of the K split
     "cfg2": int((115831 * 2.0 + 114688 * 1.0) * 1024),   # 355 MB

@@ -56,12 +56,13 @@ namespace {
 
 constexpr int DS_BN = 128;
 constexpr int DS_THREADS = 512;
-constexpr int DS_NS = 6;
 constexpr unsigned AUX_L1_MISS = 16;  // cache policy of the partial-patch loads (sc1): past the L1, served by the L2
 constexpr unsigned long long SPIN_LIMIT_TICKS = 100000000ull;  // one second of the constant 100 MHz counter (s_memrealtime)
 
-// MT = 16-row tiles of A a workgroup multiplies (2: M <= 32, 4: M <= 64)
-template <int MT>
+// MT = 16-row tiles of A a workgroup multiplies (2: M <= 32, 4: M <= 64); DS_NS = stages of the LDS ring (6: one
+// workgroup per CU with its whole K range in flight when that is short; 3: two workgroups per CU, so that one
+// streams while the other starts up or hands over -- for launches of many workgroups with long K ranges)
+template <int MT, int DS_NS>
 struct DecodeShape {
     static constexpr int RSA = 16 * MT;                 // LDS bytes per k-row of A
     static constexpr int MAT_B = KBLOCK * 128;
@@ -99,11 +100,11 @@ struct DecodeProblem {
 // Work units = (problem, strip), numbered problem-major; `units` of them.  Linear workgroup ids that
 // agree modulo 8 share an XCD: the ksplit workgroups of unit u sit at ids xcd + 8 * (grp * ksplit + split)
 // with u = grp * 8 + xcd.
-template <int MT, bool GROUPED>
+template <int MT, bool GROUPED, int DS_NS>
 __device__ __forceinline__ void decode_body(const DecodeProblem& one, const GroupTable* tab, float* mailbox, int N, int K,
                                             int strips, int units, int ksplit, int kb_per_split)
 {
-    using S = DecodeShape<MT>;
+    using S = DecodeShape<MT, DS_NS>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     auto lds = LDS_PTR(uint8_t, smem);
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -334,22 +335,22 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     store_c(sum);
 }
 
-template <int MT>
+template <int MT, int DS_NS>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int N, int K,
                     int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
-    decode_body<MT, false>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
+    decode_body<MT, false, DS_NS>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
 }
 
-template <int MT>
+template <int MT, int DS_NS>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
-    decode_body<MT, true>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
+    decode_body<MT, true, DS_NS>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
 }
 
 // records the XCC (XCD) id each workgroup of a probe grid runs on
@@ -365,6 +366,11 @@ __global__ void xcc_probe_kernel(unsigned int* out)
 }
 
 inline int row_tiles(int m) { return m <= 32 ? 2 : 4; }
+
+// Two workgroups per CU with a three-stage ring instead of one with six: one streams while the other starts up.
+// Measured on grouped launches: 64 groups x 56 strips, 16 K blocks each: 221 against 236 us; with 768-1152
+// workgroups (1.5-2.25 rounds of 512 resident ones) 1-3 % slower than three to four and a half rounds of 256.
+inline bool shallow_ring_pays(long workgroups, int kb_per_split) { return workgroups >= 2048 && kb_per_split >= 6; }
 
 }  // namespace
 
@@ -444,18 +450,16 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
     if ((ksplit - 1) * kb_per_split >= nkb)  // every split owns at least one K block
         return hipErrorInvalidValue;
     const dim3 grid(8 * ((strips + 7) / 8) * ksplit);
-    if (row_tiles(g.m) == 2) {
-        auto kern = decode_strip_kernel<2>;
-        FP8GEMM_ALLOW_LDS(kern, DecodeShape<2>::LDS);
-        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<2>::LDS, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
-                           mailbox, g.m, g.n, g.k, strips, ksplit, kb_per_split);
-    } else {
-        auto kern = decode_strip_kernel<4>;
-        FP8GEMM_ALLOW_LDS(kern, DecodeShape<4>::LDS);
-        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<4>::LDS, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
-                           mailbox, g.m, g.n, g.k, strips, ksplit, kb_per_split);
-    }
-    return hipGetLastError();
+    auto go = [&](auto kern, int lds) -> hipError_t {
+        FP8GEMM_ALLOW_LDS(kern, lds);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c, mailbox, g.m, g.n,
+                           g.k, strips, ksplit, kb_per_split);
+        return hipGetLastError();
+    };
+    const bool deep = !shallow_ring_pays((long)strips * ksplit, kb_per_split);
+    if (row_tiles(g.m) == 2)
+        return deep ? go(decode_strip_kernel<2, 6>, DecodeShape<2, 6>::LDS) : go(decode_strip_kernel<2, 3>, DecodeShape<2, 3>::LDS);
+    return deep ? go(decode_strip_kernel<4, 6>, DecodeShape<4, 6>::LDS) : go(decode_strip_kernel<4, 3>, DecodeShape<4, 3>::LDS);
 }
 
 // every group: 1 <= m <= lda <= 64 with lda a multiple of 16 (rows m .. lda-1 of a and a_scale hold zeros),
@@ -522,18 +526,17 @@ hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit
     for (int g = 0; g < tab.groups; ++g)
         mmax = tab.lda[g] > mmax ? tab.lda[g] : mmax;
     const dim3 grid((unsigned)(8 * ((units + 7) / 8) * ksplit));
-    if (row_tiles(mmax) == 2) {
-        auto kern = decode_strip_grouped_kernel<2>;
-        FP8GEMM_ALLOW_LDS(kern, DecodeShape<2>::LDS);
-        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<2>::LDS, s, tab, mailbox, n, k, strips, ksplit,
-                           kb_per_split);
-    } else {
-        auto kern = decode_strip_grouped_kernel<4>;
-        FP8GEMM_ALLOW_LDS(kern, DecodeShape<4>::LDS);
-        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), DecodeShape<4>::LDS, s, tab, mailbox, n, k, strips, ksplit,
-                           kb_per_split);
-    }
-    return hipGetLastError();
+    auto go = [&](auto kern, int lds) -> hipError_t {
+        FP8GEMM_ALLOW_LDS(kern, lds);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), lds, s, tab, mailbox, n, k, strips, ksplit, kb_per_split);
+        return hipGetLastError();
+    };
+    const bool deep = !shallow_ring_pays(units * ksplit, kb_per_split);
+    if (row_tiles(mmax) == 2)
+        return deep ? go(decode_strip_grouped_kernel<2, 6>, DecodeShape<2, 6>::LDS)
+                    : go(decode_strip_grouped_kernel<2, 3>, DecodeShape<2, 3>::LDS);
+    return deep ? go(decode_strip_grouped_kernel<4, 6>, DecodeShape<4, 6>::LDS)
+                : go(decode_strip_grouped_kernel<4, 3>, DecodeShape<4, 3>::LDS);
 }
 
 }  // namespace fp8gemm

@@ -685,7 +685,8 @@ def test_grouped_gemm_takes_more_groups_than_one_launch_holds(pkg):
                                     ([64] * 24, 512, 1024),
                                     ([16] * 64, 256, 384),
                                     ([32, 48], 576, 128),                             # one K block: nothing to split
-                                    ([16, 64, 32, 16], 7168, 512)])
+                                    ([16, 64, 32, 16], 7168, 512),
+                                    ([16] * 62 + [48, 32], 4096, 768)])              # 2048 work units: two workgroups per CU
 def test_grouped_decode_groups_equal_the_problems_one_by_one(pkg, ms, n, k):
     """groups of at most 64 rows (an MoE layer in a decode step): one launch of the decode kernel, every
     group bit-identical to a single launch of that kernel with the same K split"""
