@@ -615,22 +615,35 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
         if (differs && !placement_ok(stream))
             cfg.fused_ok = false;
     }
-    const Plan p = make_plan(g, cfg);
+    Plan p = make_plan(g, cfg);
     if (p.family < 0)
         return FP8GEMM_E_KERNEL;
-    const size_t need = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p), plan_uses_header(p));
     Workspace w{nullptr, 0, false};
-    if (need) {
-        if (explicit_ws) {
-            if (!explicit_ws->ptr || explicit_ws->bytes < need ||
-                (reinterpret_cast<uintptr_t>(explicit_ws->ptr) % 256) != 0)
-                return FP8GEMM_E_WORKSPACE;
-            w = *explicit_ws;
-        } else {
-            const int rc = acquire_workspace(need, stream, &w);
-            if (rc != FP8GEMM_OK)
-                return rc;
+    for (int attempt = 0;; ++attempt) {
+        const size_t need = p.padded ? padded_bytes(g, p) : with_header(plan_workspace_bytes(g, p), plan_uses_header(p));
+        int rc = FP8GEMM_OK;
+        if (need) {
+            if (explicit_ws) {
+                if (!explicit_ws->ptr || explicit_ws->bytes < need ||
+                    (reinterpret_cast<uintptr_t>(explicit_ws->ptr) % 256) != 0)
+                    rc = FP8GEMM_E_WORKSPACE;
+                else
+                    w = *explicit_ws;
+            } else {
+                rc = acquire_workspace(need, stream, &w);
+            }
         }
+        if (rc == FP8GEMM_OK)
+            break;
+        // A plan that adds its K splits inside the kernel needs the header; when the workspace at hand cannot
+        // hold it (a small caller-owned buffer, or none while the stream is being captured) the plan without
+        // it may still run -- cfg1-like shapes then need no workspace at all.  Not when that form was asked for.
+        if (rc != FP8GEMM_E_WORKSPACE || attempt > 0 || !cfg.fused_ok || cfg.fused_mode == 1 || !plan_uses_header(p))
+            return rc;
+        cfg.fused_ok = false;
+        p = make_plan(g, cfg);
+        if (p.family < 0)
+            return FP8GEMM_E_WORKSPACE;
     }
     const int rc = p.padded ? run_padded(g, p, w, stream) : (int)launch_plan(g, p, ws_data(w), w, stream);
     if (rc == FP8GEMM_OK) {

@@ -311,3 +311,42 @@ def test_grouped_per_call_form_from_two_threads_on_two_streams(pkg):
                             j["ms"], j["n"], j["k"], None, None, 0, j["stream"].cuda_stream)
     assert info.value.code == -4
     torch.cuda.synchronize()
+
+
+def test_plan_without_the_header_runs_when_no_workspace_can_be_had(pkg):
+    """a shape whose preferred plan adds its K splits inside the kernel (and so needs the workspace header)
+    still runs when no workspace is at hand -- a per-call entry without a buffer, the process-wide entry while
+    its stream is being captured and nothing is allocated yet -- on the plan that needs none"""
+    import torch
+    m, n, k = 1024, 512, 2048
+    assert pkg.plan(m, n, k) == "tile64x64_k2f"
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 8701)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    dev = _dev(a, b, sa, sb)
+    dc = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    _say(f"[gpu case] per-call entry without a workspace m={m} n={n} k={k}")
+    pkg.gemm_ex(*dev, dc, m, n, k, pkg.Options(flags=pkg.FLAG_WORKSPACE_ZEROED), None, 0, st)
+    torch.cuda.synchronize()
+    assert pkg.last_kernel() == "tile64x64_k1", pkg.last_kernel()
+    assert oracle.compare_bf16(dc.cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0
+    pkg.set_workspace(None, 0)
+    pkg.release()
+    dc.fill_(-1)
+    torch.cuda.synchronize()
+    _say("[gpu case] process-wide entry under capture, nothing allocated")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pkg.gemm(*dev, dc, m, n, k, torch.cuda.current_stream().cuda_stream)
+        name = pkg.last_kernel()
+    assert name == "tile64x64_k1", name
+    graph.replay()
+    torch.cuda.synchronize()
+    assert oracle.compare_bf16(dc.cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0
+    del graph
+    # with the library's workspace in place the preferred plan runs
+    pkg.gemm(*dev, dc, m, n, k, st)
+    torch.cuda.synchronize()
+    assert pkg.last_kernel() == "tile64x64_k2f", pkg.last_kernel()
+    assert oracle.compare_bf16(dc.cpu().numpy().view(np.uint16), ref, 1e-2, 1e-3)["bad"] == 0
+    pkg.release()
