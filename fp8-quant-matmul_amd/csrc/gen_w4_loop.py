@@ -297,6 +297,51 @@ def k_block(a, slots_before_first_fold):
     return this_mfma
 
 
+def verify_distances(a):
+    """The two hazards the loop keeps by counting instruction slots, checked on the emitted text over two
+    rounds of the loop: a VALU read of a block sum lies at least MFMA_RESULT_SLOTS behind the MFMA that
+    wrote it last, and a fragment read that overwrites an a-register lies at least REFILL_SLOTS behind the
+    last MFMA that reads it.  (Both distances count from the MFMA's issue, as the schedule does.)"""
+    import re
+    first = a.lines.index(".Lw4_block_%=:")
+    body = [(k, ln) for k, ln in enumerate(a.lines) if k > first]
+    seq = body + body          # the second round sees the first round's MFMAs behind it
+    cost = []                  # slots of each entry of seq
+    for k, ln in seq:
+        if ln.endswith(":") or k in a.skippable:
+            cost.append(0)
+        else:
+            cost.append(int(ln.split()[1]) + 1 if ln.startswith("s_nop") else 1)
+    mfma = re.compile(r"v_mfma\S* v\[(\d+):(\d+)\], a\[(\d+):(\d+)\], a\[(\d+):(\d+)\]")
+    fmac = re.compile(r"v_fmac_f32 v\d+, v\d+, v(\d+)$")
+    read = re.compile(r"ds_read_b64_tr_b8 a\[(\d+):(\d+)\]")
+    checked = 0
+    for pos in range(len(body), len(seq)):
+        ln = seq[pos][1]
+        need = None
+        m = fmac.match(ln)
+        if m and BLK[0] <= int(m.group(1)) < BLK[1] + 16:
+            reg = int(m.group(1))
+            need = (MFMA_RESULT_SLOTS, lambda mm: int(mm.group(1)) <= reg <= int(mm.group(2)))
+        m = read.match(ln)
+        if m:
+            lo, hi = int(m.group(1)), int(m.group(2))
+            need = (REFILL_SLOTS, lambda mm: any(int(mm.group(x)) <= hi and lo <= int(mm.group(x + 1)) for x in (3, 5)))
+        if need is None:
+            continue
+        slots = 0
+        for back in range(pos - 1, -1, -1):
+            mm = mfma.match(seq[back][1])
+            if mm and need[1](mm):
+                assert slots >= need[0], f"'{ln}' is {slots} slots behind '{seq[back][1]}', needs {need[0]}"
+                checked += 1
+                break
+            slots += cost[back]
+        else:
+            raise AssertionError(f"no MFMA found behind '{ln}'")
+    assert checked > 0
+
+
 def emit_loop(out):
     def build(tail_slots):
         a = Asm()
@@ -311,6 +356,7 @@ def emit_loop(out):
     _, tail_slots = build(0)
     a, check = build(tail_slots)
     assert check == tail_slots, "the padding of the first gap changed the tail it was computed from"
+    verify_distances(a)
     w = out.append
     w("// `count` (>= 1) K blocks of the current tile: MFMAs, folds, fragment reads, and the copies of the")
     w("// stream's next `count` blocks (offsets off_* advance by str_* per block; a stream that has run dry")
