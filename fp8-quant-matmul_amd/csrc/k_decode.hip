@@ -353,6 +353,168 @@ decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, 
     decode_body<MT, true, DS_NS>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
 }
 
+// The streaming form, for a single problem without a K split whose strips outnumber the workgroups the
+// device holds at once (N > 32768: the output projection onto a vocabulary): gridDim.x workgroups walk
+// through the strips (workgroup w takes strips w, w + gridDim.x, ...) and the K blocks of all strips of a
+// workgroup form ONE copy stream, so the first stages of the next strip are on their way while the current one
+// is multiplied and stored, instead of every strip starting from an empty ring (M = 32, N = 65536, K = 2048:
+// 23.4 against 26.3 us = 5.7 TB/s).  Same stages, same reads, same arithmetic per strip as decode_body:
+// bit-identical results.  Grouped launches gain nothing from it (64 groups x 56 strips: 225 against 220 us)
+// and keep the plain form.  (A strip's two stores per wave share the vmcnt counter with the copies and may
+// complete after younger copies; counting them as outstanding copies only makes a wait longer, never shorter.)
+template <int MT, int DS_NS>
+__device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int N, int K, int units)
+{
+    using S = DecodeShape<MT, DS_NS>;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    auto lds = LDS_PTR(uint8_t, smem);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int G = (int)gridDim.x, w = (int)blockIdx.x;
+    if (w >= units)
+        return;
+    const int nkb = K / KBLOCK;
+    const int sn = (N + KBLOCK - 1) / KBLOCK;
+    const int total = ((units - w + G - 1) / G) * nkb;  // stages of this workgroup's stream
+
+    // ---- copy side: what the strip being copied needs (see decode_body for the plan)
+    const DecodeProblem cp = one;
+    int cp_strip = 0;
+    uint32_t voff_b[2] = {0, 0}, voff_a = 0, voff_sa = 0, voff_sb = 0;
+    auto enter_copy_unit = [&](int unit) __attribute__((always_inline)) {
+        cp_strip = unit;
+        const int n0 = cp_strip * DS_BN;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int cc = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
+            const bool ok = n0 + 16 * cc < N;
+            voff_b[q] = ok ? (uint32_t)((16 * wave + 8 * q + (lane >> 3)) * N + n0 + 16 * cc) : 0x80000000u;
+        }
+        voff_sa = lane < cp.lda ? (uint32_t)(lane * 4) : 0x80000000u;
+        voff_sb = lane == 0 ? (uint32_t)(cp_strip * 4) : 0x80000000u;
+        if (MT == 2) {
+            const int cc = (lane & 1) ^ ((lane >> 4) & 1);
+            voff_a = 16 * cc < cp.lda ? (uint32_t)((32 * wave + (lane >> 1)) * cp.lda + 16 * cc) : 0x80000000u;
+        } else {
+            const int cc = (lane & 3) ^ ((lane >> 4) & 3);
+            voff_a = 16 * cc < cp.lda ? (uint32_t)((16 * wave + (lane >> 2)) * cp.lda + 16 * cc) : 0x80000000u;
+        }
+    };
+    auto issue_stage = [&](int slot, int kb) __attribute__((always_inline)) {
+        const uint32_t a_bytes = (uint32_t)cp.lda * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
+        const uint32_t stage = lds_base + (uint32_t)(slot * S::STAGE);
+        const uint32_t skip_b = (uint32_t)kb * KBLOCK * (uint32_t)N;
+        const uint32_t skip_a = (uint32_t)kb * KBLOCK * (uint32_t)cp.lda;
+        const v4i rb = make_rsrc_words(cp.b + skip_b, b_bytes - skip_b);
+        lds_dma16(rb, voff_b[0], stage + (uint32_t)((2 * wave) * 1024));
+        lds_dma16(rb, voff_b[1], stage + (uint32_t)((2 * wave + 1) * 1024));
+        const int scale_wave = MT == 2 ? wave - 4 : wave;
+        if (MT == 4 || wave < 4)
+            lds_dma16(make_rsrc_words(cp.a + skip_a, a_bytes - skip_a), voff_a, stage + S::MAT_B + (uint32_t)(wave * 1024));
+        if (scale_wave == 0)
+            lds_dma4(make_rsrc_words(cp.a_scale + (size_t)kb * cp.lda, (uint32_t)cp.lda * 4u), voff_sa, stage + S::SA_OFF);
+        else if (scale_wave > 0)
+            lds_dma4(make_rsrc_words(cp.b_scale + (size_t)kb * sn, (uint32_t)sn * 4u), voff_sb, stage + S::SB_OFF);
+    };
+    int cp_kb = 0, cp_unit = w, cp_slot = 0, issued = 0;
+    auto issue_next = [&]() __attribute__((always_inline)) {
+        if (issued >= total)
+            return;
+        if (cp_kb == 0)
+            enter_copy_unit(cp_unit);
+        issue_stage(cp_slot, cp_kb);
+        ++issued;
+        cp_slot = cp_slot == DS_NS - 1 ? 0 : cp_slot + 1;
+        if (++cp_kb == nkb) {
+            cp_kb = 0;
+            cp_unit += G;
+        }
+    };
+
+    // ---- multiply side
+    const int g4 = lane >> 4, i16 = lane & 15;
+    const uint32_t addr_b = (uint32_t)((8 * g4 + (i16 >> 1)) * 128 + ((wave ^ ((4 * g4 + (i16 >> 2)) & 7)) * 16) +
+                                       (i16 & 1) * 8);
+    const uint32_t addr_a = (uint32_t)(S::MAT_B + (8 * g4 + (i16 >> 1)) * S::RSA + (i16 & 1) * 8);
+    const int swz_a = MT == 2 ? (g4 & 1) : ((2 * g4 + (i16 >> 3)) & 3);
+    auto read_frag = [&](uint32_t addr, int step) __attribute__((always_inline)) -> v8i {
+        v2i r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr));
+        v2i r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr + step));
+        v2i r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr + 2 * step));
+        v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr + 3 * step));
+        return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+    };
+    v4f acc[MT];
+    const DecodeProblem mp = one;
+    const int mtiles = (mp.M + 15) >> 4;
+    int mp_strip = 0;
+
+#pragma unroll
+    for (int p = 0; p < DS_NS - 1; ++p)
+        issue_next();
+    int slot = 0, kb = 0, unit = w;
+    for (int t = 0; t < total; ++t) {
+        const int younger = total - 1 - t < DS_NS - 2 ? total - 1 - t : DS_NS - 2;
+        switch (younger) {
+        case 0: ds_wait_vmcnt<0>(); break;
+        case 1: ds_wait_vmcnt<S::COPIES>(); break;
+        case 2: ds_wait_vmcnt<2 * S::COPIES>(); break;
+        case 3: ds_wait_vmcnt<3 * S::COPIES>(); break;
+        default: ds_wait_vmcnt<4 * S::COPIES>(); break;
+        }
+        __syncthreads();  // everyone's copies of stage t landed; the slot of stage t - 1 is no longer read
+        issue_next();     // stage t + DS_NS - 1 goes into the slot of stage t - 1
+        if (kb == 0) {
+            mp_strip = unit;
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+        }
+        const uint32_t so = (uint32_t)(slot * S::STAGE);
+        const v8i fb = read_frag(so + addr_b, 32 * 128);
+        const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            if (i < mtiles) {
+                const v8i fa = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
+                const float sa = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
+                const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    fb, fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                const float sc = sa * sb;
+                acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]),
+                               fmaf(sc, blk[2], acc[i][2]), fmaf(sc, blk[3], acc[i][3])};
+            }
+        }
+        slot = slot == DS_NS - 1 ? 0 : slot + 1;
+        if (++kb == nkb) {
+            // a lane holds C[16*i + (lane & 15)][n0 + 16*wave + 4*(lane >> 4) + 0..3]
+            const int ncol = mp_strip * DS_BN + 16 * wave + 4 * g4;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const int mrow = 16 * i + i16;
+                if (mrow < mp.M && ncol < N) {
+                    uint2 pk;
+                    pk.x = pack_bf16x2(acc[i][0], acc[i][1]);
+                    pk.y = pack_bf16x2(acc[i][2], acc[i][3]);
+                    *reinterpret_cast<uint2*>(mp.c + (size_t)mrow * N + ncol) = pk;
+                }
+            }
+            kb = 0;
+            unit += G;
+        }
+    }
+}
+
+template <int MT, int DS_NS>
+__global__ void __launch_bounds__(DS_THREADS)
+decode_stream_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
+                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, int M, int N, int K, int strips)
+{
+    const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
+    decode_stream_body<MT, DS_NS>(one, N, K, strips);
+}
+
 // records the XCC (XCD) id each workgroup of a probe grid runs on
 constexpr int XCC_PROBE = 256;
 static __device__ unsigned int xcc_probe_out[XCC_PROBE];
@@ -366,6 +528,10 @@ __global__ void xcc_probe_kernel(unsigned int* out)
 }
 
 inline int row_tiles(int m) { return m <= 32 ? 2 : 4; }
+
+// the streaming form: ring depth and workgroups (one per CU with six stages)
+constexpr int STREAM_NS = 6;
+constexpr int STREAM_WORKGROUPS = 256;
 
 // Two workgroups per CU with a three-stage ring instead of one with six: one streams while the other starts up.
 // Measured on grouped launches: 64 groups x 56 strips, 16 K blocks each: 221 against 236 us; with 768-1152
@@ -456,6 +622,16 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
                            g.k, strips, ksplit, kb_per_split);
         return hipGetLastError();
     };
+    if (ksplit == 1 && strips > STREAM_WORKGROUPS) {  // more units than resident workgroups: one copy stream per workgroup
+        auto stream = [&](auto kern, int lds) -> hipError_t {
+            FP8GEMM_ALLOW_LDS(kern, lds);
+            hipLaunchKernelGGL(kern, dim3(STREAM_WORKGROUPS), dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
+                               g.m, g.n, g.k, strips);
+            return hipGetLastError();
+        };
+        return row_tiles(g.m) == 2 ? stream(decode_stream_kernel<2, STREAM_NS>, DecodeShape<2, STREAM_NS>::LDS)
+                                   : stream(decode_stream_kernel<4, STREAM_NS>, DecodeShape<4, STREAM_NS>::LDS);
+    }
     const bool deep = !shallow_ring_pays((long)strips * ksplit, kb_per_split);
     if (row_tiles(g.m) == 2)
         return deep ? go(decode_strip_kernel<2, 6>, DecodeShape<2, 6>::LDS) : go(decode_strip_kernel<2, 3>, DecodeShape<2, 3>::LDS);

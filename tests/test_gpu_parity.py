@@ -240,7 +240,10 @@ def test_skinny_kernel_with_the_k_range_split_over_workgroups(pkg, m, n, k, kspl
 DECODE_STRIP_CASES = [(32, 7168, 2048, 4), (16, 7168, 2048, 4), (32, 7168, 2048, 1), (32, 576, 1024, 3),
                       (32, 1040, 2048, 16), (16, 96, 512, 2), (32, 128, 128, 1), (32, 4608, 7168, 7),
                       (16, 1536, 1536, 12), (32, 2048, 384, 3), (32, 16384, 1024, 4), (16, 16, 2048, 6),
-                      (32, 7168, 7168, 8)]
+                      (32, 7168, 7168, 8),
+                      # more strips than the device holds workgroups, no K split: the streaming form (a workgroup
+                      # walks through several strips, one copy stream); ragged last strip; a single K block
+                      (16, 33040, 384, 1), (32, 40960, 256, 1), (48, 33024, 128, 1)]
 
 
 @pytest.mark.parametrize("m,n,k,ksplit", DECODE_STRIP_CASES)
