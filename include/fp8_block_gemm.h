@@ -161,7 +161,10 @@ typedef struct fp8gemm_options {
  * launching a reduction kernel ("decode128_kN", "..._kNf") hand their partial results over through it (a
  * mailbox of 16 MiB) and leave all of it zero again after every call; without the flag a per-call workspace
  * only gets the two-kernel plans.
- * The process-wide workspace and fp8_block_gemm_noalloc's array always have a zeroed header. */
+ * The process-wide workspace and fp8_block_gemm_noalloc's array always have a zeroed header.  Calls that
+ * share a workspace and overlap on the device (which the contract forbids) can leave the header non-zero
+ * and later results wrong: zero it again before the next use (fp8_block_gemm_release() drops the
+ * library-owned buffer, whose successor starts out zeroed). */
 #define FP8GEMM_FLAG_WORKSPACE_ZEROED 1
 #define FP8GEMM_WORKSPACE_HEADER_BYTES (16u << 20)
 int fp8_block_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale, void* c,
@@ -199,9 +202,11 @@ size_t fp8_block_gemm_grouped_workspace_bytes_ex(int groups, const int* m, int n
  * A plan that needs more than that returns FP8GEMM_E_WORKSPACE (ask fp8_block_gemm_workspace_bytes /
  * _ex beforehand; plans that neither split K nor pad need nothing and always fit).  All calls on one
  * GPU share that GPU's array: calls that use it and overlap on the device (different streams) race, as
- * with the process-wide workspace.  Nothing in it has to start at zero: every plan writes what it later
- * reads.  The first call on a device looks the array's address up (hipGetSymbolAddress); make that call
- * outside a stream capture.  This entry point has no counterpart in the reference. */
+ * with the process-wide workspace.  The caller clears nothing: the array starts out zero, the plans that
+ * use its first FP8GEMM_WORKSPACE_HEADER_BYTES (the mailbox of the K splits) leave them zero, every other
+ * plan writes what it later reads.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make that call outside a stream capture.  This entry point has no counterpart in
+ * the reference. */
 #define FP8GEMM_NOALLOC_MAX_BYTES (32u << 20)
 int fp8_block_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
                            void* c, int m, int n, int k, void* stream);
