@@ -477,6 +477,48 @@ def test_nan_and_zero_scale_do_not_leak_into_other_elements(pkg):
     _assert_close(np.delete(got, 7, axis=0), np.delete(ref, 7, axis=0), name)
 
 
+@pytest.mark.parametrize("m,n,k,kw", [(32, 1536, 1024, dict(kernel=4, variant=1, ksplit=4)),
+                                      (64, 640, 512, dict(kernel=4, variant=1, ksplit=2)),
+                                      (256, 384, 1024, dict(kernel=3, variant=4, ksplit=4, fused=1)),
+                                      (256, 384, 768, dict(kernel=3, variant=2, ksplit=3, fused=1))])
+def test_special_values_through_the_mailbox_plans(pkg, m, n, k, kw):
+    """plans whose K splits meet in the mailbox write +0.0 as -0.0 so that no word is zero: all-zero operands
+    still give +0.0 bit for bit, one-hot operands (most partial sums are zero) the exact single products, a NaN
+    stays in its row, and the mailbox is zero again afterwards (the next launch is right)"""
+    nkb = k // 128
+    sn = (n + 127) // 128
+    rng = np.random.RandomState(m + n + k)
+    sa = rng.uniform(1, 2, (nkb, m)).astype(np.float32)
+    sb = rng.uniform(1, 2, (nkb, sn)).astype(np.float32)
+    zeros_a, zeros_b = np.zeros((k, m), np.uint8), np.zeros((k, n), np.uint8)
+    got, name = _run(pkg, zeros_a, zeros_b, sa, sb, m, n, k, **kw)
+    assert (got == 0).all(), f"{name}: all-zero operands must give +0.0 everywhere"
+    a, b = zeros_a.copy(), zeros_b.copy()
+    pts = [(0, 0, 0), (m - 1, n - 1, k - 1), (m // 2 + 1, n // 3, k // 2), (3, n - 2, 129), (m - 2, 5, k - 130)]
+    for (mi, ni, ki) in pts:
+        a[ki, mi] = 0x44   # 3.0
+        b[ki, ni] = 0xB8   # -1.0
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, **kw)
+    assert np.array_equal(got, ref), name
+    assert np.count_nonzero(ref) == len(pts)
+    a2, b2, sa2, sb2 = oracle.make_inputs(m, n, k, 4100 + m)
+    a2[k - 3, 7] = 0x7F     # NaN in row 7, in the last split's K range
+    a2[2, 11] = 0xFF        # NaN in row 11, in the first split's
+    ref = oracle.ref_gemm(a2, b2, sa2, sb2, m, n, k)
+    got, name = _run(pkg, a2, b2, sa2, sb2, m, n, k, **kw)
+    gf = oracle.bf16_decode(got)
+    assert np.isnan(gf[7]).all() and np.isnan(gf[11]).all()
+    keep = np.delete(np.arange(m), [7, 11])
+    assert not np.isnan(gf[keep]).any()
+    _assert_close(got[keep], ref[keep], name)
+    # and the launch after those finds a clean mailbox
+    a3, b3, sa3, sb3 = oracle.make_inputs(m, n, k, 4200 + m)
+    got, name = _run(pkg, a3, b3, sa3, sb3, m, n, k, **kw)
+    _assert_close(got, oracle.ref_gemm(a3, b3, sa3, sb3, m, n, k), name)
+    _assert_every_element(got, a3, b3, sa3, sb3, m, n, k, name)
+
+
 # ------------------------------------------------------------------ converter, host launcher, workspace, drivers
 def test_convert_kernel_is_bit_exact(pkg):
     import torch
