@@ -519,6 +519,56 @@ def test_special_values_through_the_mailbox_plans(pkg, m, n, k, kw):
     _assert_every_element(got, a3, b3, sa3, sb3, m, n, k, name)
 
 
+def test_mailbox_plans_back_to_back_in_random_order(pkg):
+    """three seconds of launches of the plans that hand their K splits over through the mailbox, shapes in random
+    order and without synchronisation in between (every launch finds the zeros the one before left behind):
+    every result equals that plan's first one bit for bit"""
+    import time
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    cases = [(32, 7168, 2048, pkg.KERNEL_SKINNY, 1, 4), (16, 1536, 7168, pkg.KERNEL_SKINNY, 1, 8),
+             (1024, 512, 2048, pkg.KERNEL_SPLITK, 4, 2), (2048, 576, 7168, pkg.KERNEL_SPLITK, 2, 3),
+             (512, 512, 4096, pkg.KERNEL_SPLITK, 4, 4), (48, 1536, 2048, pkg.KERNEL_SKINNY, 1, 6)]
+    prep = []
+    pkg.set_fused_reduction(1)
+    try:
+        for (m, n, k, ker, v, ks) in cases:
+            a, b, sa, sb = oracle.make_inputs(m, n, k, 31 + m + n + k)
+            dev = _dev(a, b, sa, sb)
+            c = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+            pkg.select(ker)
+            pkg.force_config(v, ks)
+            pkg.gemm(*dev, c, m, n, k, st)
+            torch.cuda.synchronize()
+            name = pkg.last_kernel()
+            assert name.startswith("decode128_k") or name.endswith("f"), name
+            _assert_close(c.cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), name)
+            prep.append((m, n, k, ker, v, ks, dev, c, c.clone(), name))
+        _say(f"[gpu case] mailbox plans back to back: {[p[9] for p in prep]}")
+        rs = np.random.RandomState(5)
+        t0 = time.time()
+        launches = 0
+        while time.time() - t0 < 3.0:
+            outs = []
+            for i in rs.permutation(len(prep)):
+                m, n, k, ker, v, ks, dev, c, good, name = prep[i]
+                pkg.select(ker)
+                pkg.force_config(v, ks)
+                for _ in range(int(rs.randint(1, 6))):
+                    c.fill_(0x7FC1)
+                    pkg.gemm(*dev, c, m, n, k, st)
+                    launches += 1
+                outs.append((i, c.clone()))
+            torch.cuda.synchronize()
+            for i, o in outs:
+                assert torch.equal(o, prep[i][8]), f"{prep[i][9]} after {launches} launches"
+        assert launches > 1000
+    finally:
+        pkg.select(0)
+        pkg.force_config(-1, 0)
+        pkg.set_fused_reduction(-1)
+
+
 # ------------------------------------------------------------------ converter, host launcher, workspace, drivers
 def test_convert_kernel_is_bit_exact(pkg):
     import torch
