@@ -329,8 +329,8 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             p.family = -1;
             return p;
         }
-        // rows without 16-byte alignment: the padded problem (its four extra launches cost
-        // about 12 us; the scalar kernel, one dependent load after the other, takes 30 us for
+        // rows without 16-byte alignment: the padded problem (its one or two extra launches cost
+        // about 5 us; the scalar kernel, one dependent load after the other, takes 30 us for
         // K = 128 already), unless padding pushes an operand past the size limit
         const long long m16 = (g.m + 15) & ~15, n16 = (g.n + 15) & ~15, lim = 0x7FFFFFFFll;
         if (m16 * g.k > lim || n16 * g.k > lim || m16 * n16 > lim)
@@ -555,20 +555,23 @@ int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t
         return FP8GEMM_E_WORKSPACE;
     uint8_t* base = reinterpret_cast<uint8_t*>(ws_data(w));
     const int nkb = g.k / 128;
-    hipError_t e = hipSuccess;
+    // every operand that needs a padded copy, in one launch
+    PadJobs jobs;
+    jobs.count = 0;
     if (L.a) {
-        e = launch_pad_bytes(g.a, base + L.off_a, g.k, g.m, m16, stream);
+        jobs.job[jobs.count++] = PadJob{g.a, base + L.off_a, g.k, g.m, m16, 0};
         gp.a = base + L.off_a;
     }
-    if (e == hipSuccess && L.as) {
+    if (L.as) {
         float* as = reinterpret_cast<float*>(base + L.off_as);
-        e = launch_pad_floats(g.a_scale, as, nkb, g.m, m16, stream);
+        jobs.job[jobs.count++] = PadJob{g.a_scale, as, nkb, g.m, m16, 1};
         gp.a_scale = as;
     }
-    if (e == hipSuccess && L.b) {
-        e = launch_pad_bytes(g.b, base + L.off_b, g.k, g.n, gp.n, stream);
+    if (L.b) {
+        jobs.job[jobs.count++] = PadJob{g.b, base + L.off_b, g.k, g.n, gp.n, 0};
         gp.b = base + L.off_b;
     }
+    hipError_t e = launch_pad_jobs(jobs, stream);
     if (L.c)
         gp.c = reinterpret_cast<uint16_t*>(base + L.off_c);
     if (e == hipSuccess)

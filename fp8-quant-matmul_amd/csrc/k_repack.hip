@@ -128,6 +128,17 @@ __global__ void __launch_bounds__(256) repack_batched_kernel(const RepackTable t
                        (size_t)blockIdx.x * blockDim.x + threadIdx.x);
 }
 
+// up to PadJobs::MAX padding copies of either kind in one launch, one per blockIdx.y
+__global__ void __launch_bounds__(256) pad_jobs_kernel(const PadJobs jobs)
+{
+    const PadJob& j = jobs.job[blockIdx.y];
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j.floats)
+        pad_piece_floats(static_cast<const float*>(j.src), static_cast<float*>(j.dst), j.rows, j.ld_src, j.ld_dst, idx);
+    else
+        pad_piece_bytes(static_cast<const uint8_t*>(j.src), static_cast<uint8_t*>(j.dst), j.rows, j.ld_src, j.ld_dst, idx);
+}
+
 template <int KIND>
 hipError_t launch_repack(const void* src, void* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
 {
@@ -158,14 +169,21 @@ hipError_t launch_repack_batched(const RepackTable& tab, hipStream_t s)
 
 }  // namespace
 
-hipError_t launch_pad_bytes(const uint8_t* src, uint8_t* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
+hipError_t launch_pad_jobs(const PadJobs& jobs, hipStream_t s)
 {
-    return launch_repack<REPACK_PAD_BYTES>(src, dst, rows, ld_src, ld_dst, s);
-}
-
-hipError_t launch_pad_floats(const float* src, float* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
-{
-    return launch_repack<REPACK_PAD_FLOATS>(src, dst, rows, ld_src, ld_dst, s);
+    if (jobs.count < 0 || jobs.count > PadJobs::MAX)
+        return hipErrorInvalidValue;
+    size_t most = 0;
+    for (int i = 0; i < jobs.count; ++i) {
+        const PadJob& j = jobs.job[i];
+        const size_t pieces = j.floats ? repack_pieces<REPACK_PAD_FLOATS>(j.rows, j.ld_dst)
+                                       : repack_pieces<REPACK_PAD_BYTES>(j.rows, j.ld_dst);
+        most = pieces > most ? pieces : most;
+    }
+    if (most == 0)
+        return hipSuccess;
+    hipLaunchKernelGGL(pad_jobs_kernel, dim3((unsigned)((most + 255) / 256), (unsigned)jobs.count), dim3(256), 0, s, jobs);
+    return hipGetLastError();
 }
 
 hipError_t launch_crop_bf16(const uint16_t* src, uint16_t* dst, int m, int n, int ld_src, hipStream_t s)

@@ -111,13 +111,24 @@ hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit
 // 0 = they do not, or it could not be looked at; -1 = not looked at yet and may_probe is false
 int xcd_placement_confirmed(bool may_probe);
 
-// rows of ld_src elements copied into rows of ld_dst >= ld_src elements, the rest zero (dst
-// 16-byte aligned, ld_dst a multiple of 16 bytes); the m x n corner of a bf16 matrix with
-// ld_src elements per row copied into a dense one
-hipError_t launch_pad_bytes(const uint8_t* src, uint8_t* dst, int rows, int ld_src, int ld_dst, hipStream_t s);
-hipError_t launch_pad_floats(const float* src, float* dst, int rows, int ld_src, int ld_dst, hipStream_t s);
+// Padding: rows of ld_src elements copied into rows of ld_dst >= ld_src elements, the rest zero (dst
+// 16-byte aligned, ld_dst a multiple of 16 bytes).  Cropping: the m x n corner of a bf16 matrix with
+// ld_src elements per row copied into a dense one.
 hipError_t launch_crop_bf16(const uint16_t* src, uint16_t* dst, int m, int n, int ld_src, hipStream_t s);
-// the same for several matrices in one launch (the table travels by value in the kernel
+// the padding copies of one problem (bytes of a and b, fp32 values of a_scale) in one launch
+struct PadJob {
+    const void* src;
+    void* dst;
+    int rows, ld_src, ld_dst;
+    int floats;  // 0 = bytes (ld_dst a multiple of 16), 1 = fp32 values (ld_dst a multiple of 4)
+};
+struct PadJobs {
+    static constexpr int MAX = 4;
+    PadJob job[MAX];
+    int count;
+};
+hipError_t launch_pad_jobs(const PadJobs& jobs, hipStream_t s);
+// one kind of copy for several matrices in one launch (the table travels by value in the kernel
 // arguments).  Padding: rows x ld_src -> rows x ld_dst.  Cropping: rows = m, ld_src = elements
 // per source row, ld_dst = n.
 struct RepackTable {

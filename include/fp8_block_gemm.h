@@ -69,8 +69,8 @@ extern "C" {
  * same argument order and meaning.  Any m, n > 0 and k % 128 == 0.  The MFMA kernels take
  * m % 16 == 0, n % 16 == 0 and 16-byte aligned a, b, a_scale, c as they are; for anything else
  * the library copies the operands concerned into zero-padded buffers in its workspace, runs
- * there and copies c's m x n corner out (plans named "padded_...": four small extra launches,
- * about 2 bytes of extra traffic per operand byte).  The reference requires M, N % 64 (32) == 0
+ * there and copies c's m x n corner out (plans named "padded_...": one extra launch for the copies and
+ * one for c's corner, about 2 bytes of extra traffic per operand byte).  The reference requires M, N % 64 (32) == 0
  * and reads out of bounds otherwise (mn_large.hip:16). */
 int fp8_block_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                    void* c, int m, int n, int k);
