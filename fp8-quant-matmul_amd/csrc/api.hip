@@ -827,9 +827,7 @@ int run_grouped_table(const GroupTable& tab, int n, int k, bool decode, hipStrea
     }
     hipError_t e = hipSuccess;
     if (padded) {
-        e = launch_pad_bytes_batched(ta, s);
-        if (e == hipSuccess)
-            e = launch_pad_floats_batched(tas, s);
+        e = launch_pad_pair_batched(ta, tas, s);
         if (e == hipSuccess && pad_b)
             e = launch_pad_bytes_batched(tb, s);
     }

@@ -139,6 +139,17 @@ __global__ void __launch_bounds__(256) pad_jobs_kernel(const PadJobs jobs)
         pad_piece_bytes(static_cast<const uint8_t*>(j.src), static_cast<uint8_t*>(j.dst), j.rows, j.ld_src, j.ld_dst, idx);
 }
 
+// the byte copies (blockIdx.z = 0) and the fp32 copies (blockIdx.z = 1) of several problems in one launch
+__global__ void __launch_bounds__(256) pad_pair_batched_kernel(const RepackTable bytes, const RepackTable floats)
+{
+    const int g = blockIdx.y;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (blockIdx.z == 0)
+        repack_piece<REPACK_PAD_BYTES>(bytes.src[g], bytes.dst[g], bytes.rows[g], bytes.ld_src[g], bytes.ld_dst[g], idx);
+    else
+        repack_piece<REPACK_PAD_FLOATS>(floats.src[g], floats.dst[g], floats.rows[g], floats.ld_src[g], floats.ld_dst[g], idx);
+}
+
 template <int KIND>
 hipError_t launch_repack(const void* src, void* dst, int rows, int ld_src, int ld_dst, hipStream_t s)
 {
@@ -191,14 +202,27 @@ hipError_t launch_crop_bf16(const uint16_t* src, uint16_t* dst, int m, int n, in
     return launch_repack<REPACK_CROP_BF16>(src, dst, m, ld_src, n, s);
 }
 
+hipError_t launch_pad_pair_batched(const RepackTable& bytes, const RepackTable& floats, hipStream_t s)
+{
+    if (bytes.groups < 1 || bytes.groups > RepackTable::MAX_GROUPS || floats.groups != bytes.groups)
+        return hipErrorInvalidValue;
+    size_t most = 0;
+    for (int g = 0; g < bytes.groups; ++g) {
+        const size_t pb = repack_pieces<REPACK_PAD_BYTES>(bytes.rows[g], bytes.ld_dst[g]);
+        const size_t pf = repack_pieces<REPACK_PAD_FLOATS>(floats.rows[g], floats.ld_dst[g]);
+        most = pb > most ? pb : most;
+        most = pf > most ? pf : most;
+    }
+    if (most == 0)
+        return hipSuccess;
+    hipLaunchKernelGGL(pad_pair_batched_kernel, dim3((unsigned)((most + 255) / 256), (unsigned)bytes.groups, 2), dim3(256), 0, s,
+                       bytes, floats);
+    return hipGetLastError();
+}
+
 hipError_t launch_pad_bytes_batched(const RepackTable& tab, hipStream_t s)
 {
     return launch_repack_batched<REPACK_PAD_BYTES>(tab, s);
-}
-
-hipError_t launch_pad_floats_batched(const RepackTable& tab, hipStream_t s)
-{
-    return launch_repack_batched<REPACK_PAD_FLOATS>(tab, s);
 }
 
 hipError_t launch_crop_bf16_batched(const RepackTable& tab, hipStream_t s)

@@ -141,7 +141,8 @@ struct RepackTable {
     int groups;
 };
 hipError_t launch_pad_bytes_batched(const RepackTable& tab, hipStream_t s);
-hipError_t launch_pad_floats_batched(const RepackTable& tab, hipStream_t s);
+// byte copies (a of every group) and fp32 copies (a_scale of every group) in one launch; same group count
+hipError_t launch_pad_pair_batched(const RepackTable& bytes, const RepackTable& floats, hipStream_t s);
 hipError_t launch_crop_bf16_batched(const RepackTable& tab, hipStream_t s);
 
 // fp32 -> e4m3fn (check.cu:17-22)
