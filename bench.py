@@ -416,6 +416,23 @@ def main():
                 out["kernel"] = pkg.last_kernel()
         return out
 
+    def decode_rows_report(steps, warmup, rows=(1, 8, 16, 24, 32), dn=7168, dk=2048):
+        """cfg5's weight matrix against decode batches of other sizes, among them row counts off the 16-byte
+        grid (the decode kernel takes those as they are): latency with B in the caches and with B from HBM"""
+        out = []
+        for m in rows:
+            shape, host, dev, dc = prepare((m, dn, dk, 3100 + m))
+            step(dev, dc, shape)
+            torch.cuda.synchronize()
+            par = parity(host, dc, shape, npts=2048)
+            _, ev_ms = timed(dev, dc, shape, steps, warmup)
+            rot_us, _ = rotating_operand_us(dev, dc, shape)
+            _, byts = algorithmic_work(*shape)
+            out.append({"m": m, "n": dn, "k": dk, "kernel": pkg.last_kernel(), "latency_us": round(ev_ms * 1e3, 2),
+                        "hbm_rotating_us": round(rot_us, 2), "hbm_rotating_gbs": round(byts / rot_us * 1e-3, 1),
+                        "parity_pass": par["pass"]})
+        return out
+
     def grouped_decode_report(steps, warmup, experts=64, gn=7168, gk=2048, on_grid=False):
         """an MoE layer in a decode step: `experts` problems of 1 to 64 rows each (seeded), every expert with
         its own weights (64 x 14.7 MB: streamed from HBM on every launch).  One grouped call (one launch of
@@ -501,9 +518,10 @@ def main():
         grouped["off_grid"] = grouped_report(max(30, args.steps), args.warmup,
                                              ms=(509, 1027, 771, 1533, 250, 2051, 1023, 1028))
     grouped_decode = None
-    if not args.no_shapes:   # 64 experts of 1..64 rows (padded copies of A), and the same on the 16-row grid
+    if not args.no_shapes:   # 64 experts of 1..64 rows, and the same on the 16-row grid
         grouped_decode = grouped_decode_report(max(20, args.steps), args.warmup)
         grouped_decode["on_grid"] = grouped_decode_report(max(20, args.steps), args.warmup, on_grid=True)
+    decode_rows = None if args.no_shapes else decode_rows_report(max(20, args.steps), args.warmup)
     host_boundary = None if args.no_shapes else host_boundary_report()
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
@@ -566,6 +584,7 @@ def main():
         "vendor_plain_fp8_gemm": vendor,
         "grouped": grouped,
         "grouped_decode": grouped_decode,
+        "decode_rows": decode_rows,
         "host_boundary": host_boundary,
         "device": device,
     }

@@ -56,20 +56,26 @@ namespace {
 
 constexpr int DS_BN = 128;
 constexpr int DS_THREADS = 512;
+constexpr int RAGGED4_NS = 4;  // ring stages of the four-row-tile kernel that also holds A's packed slabs
 constexpr unsigned AUX_L1_MISS = 16;  // cache policy of the partial-patch loads (sc1): past the L1, served by the L2
 constexpr unsigned long long SPIN_LIMIT_TICKS = 100000000ull;  // one second of the constant 100 MHz counter (s_memrealtime)
 
 // MT = 16-row tiles of A a workgroup multiplies (2: M <= 32, 4: M <= 64); DS_NS = stages of the LDS ring (6: one
 // workgroup per CU with its whole K range in flight when that is short; 3: two workgroups per CU, so that one
 // streams while the other starts up or hands over -- for launches of many workgroups with long K ranges)
-template <int MT, int DS_NS>
+// RAGGED = the row count is not a multiple of 16, so that k-rows of A do not start on 16-byte boundaries: a stage
+// then also holds the K block's slab of A as it lies in memory, [128][M] bytes packed -- which does start on a
+// 16-byte boundary, 128 * M * kb bytes into A -- and the threads spread it into the padded rows the reads expect.
+template <int MT, int DS_NS, bool RAGGED = false>
 struct DecodeShape {
     static constexpr int RSA = 16 * MT;                 // LDS bytes per k-row of A
     static constexpr int MAT_B = KBLOCK * 128;
     static constexpr int MAT_A = KBLOCK * RSA;
     static constexpr int SA_OFF = MAT_B + MAT_A;        // up to 64 a_scale floats
     static constexpr int SB_OFF = SA_OFF + 256;         // 1 float (every wave that brings it writes the same bytes)
-    static constexpr int STAGE = SB_OFF + 256;
+    static constexpr int PACK_OFF = SB_OFF + 256;       // RAGGED: the packed slab of A, up to MAT_A bytes, and 16
+    // bytes the last row's reads may run into; stages start on 512-byte boundaries
+    static constexpr int STAGE = RAGGED ? (PACK_OFF + MAT_A + 16 + 511) / 512 * 512 : PACK_OFF;
     static constexpr int LDS = DS_NS * STAGE;
     // copy instructions per wave and stage: two of B, then A / scales
     //   MT = 2: waves 0..3 A (32 rows x 32 B each), wave 4 a_scale, waves 5..7 b_scale
@@ -77,7 +83,7 @@ struct DecodeShape {
     static constexpr int COPIES = MT == 2 ? 3 : 4;
     static_assert(MT == 2 || MT == 4, "two or four row tiles");
     static_assert(LDS <= 160 * 1024, "ring exceeds the LDS");
-    static_assert(COPIES * (DS_NS - 2) < 64, "vmcnt is a 6-bit field");
+    static_assert(COPIES * (DS_NS - 1) < 64, "vmcnt is a 6-bit field");
 };
 
 template <int N>
@@ -100,11 +106,11 @@ struct DecodeProblem {
 // Work units = (problem, strip), numbered problem-major; `units` of them.  Linear workgroup ids that
 // agree modulo 8 share an XCD: the ksplit workgroups of unit u sit at ids xcd + 8 * (grp * ksplit + split)
 // with u = grp * 8 + xcd.
-template <int MT, bool GROUPED, int DS_NS>
+template <int MT, bool GROUPED, int DS_NS, bool RAGGED>
 __device__ __forceinline__ void decode_body(const DecodeProblem& one, const GroupTable* tab, float* mailbox, int N, int K,
                                             int strips, int units, int ksplit, int kb_per_split)
 {
-    using S = DecodeShape<MT, DS_NS>;
+    using S = DecodeShape<MT, DS_NS, RAGGED>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     auto lds = LDS_PTR(uint8_t, smem);
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -154,7 +160,11 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     const uint32_t voff_sa = lane < lda ? (uint32_t)(lane * 4) : 0x80000000u;
     const uint32_t voff_sb = lane == 0 ? (uint32_t)(strip * 4) : 0x80000000u;
     uint32_t voff_a;
-    if (MT == 2) {
+    if (RAGGED) {
+        // the K block's slab of A, 128 * M contiguous bytes, in 16-byte pieces: piece 64 * wave + lane
+        const int piece = 64 * wave + lane;
+        voff_a = 16 * piece < KBLOCK * lda ? (uint32_t)(16 * piece) : 0x80000000u;
+    } else if (MT == 2) {
         const int cc = (lane & 1) ^ ((lane >> 4) & 1);
         voff_a = 16 * cc < lda ? (uint32_t)((32 * wave + (lane >> 1)) * lda + 16 * cc) : 0x80000000u;
     } else {
@@ -171,12 +181,65 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         lds_dma16(rb, voff_b[0], stage + (uint32_t)((2 * wave) * 1024));
         lds_dma16(rb, voff_b[1], stage + (uint32_t)((2 * wave + 1) * 1024));
         const int scale_wave = MT == 2 ? wave - 4 : wave;  // 0: a_scale, 1..: b_scale, below 0: A (two row tiles)
-        if (MT == 4 || wave < 4)
+        if (RAGGED) {
+            // the slab of the K block after this one, into the next slot: it has landed with this stage, one
+            // stage before it is multiplied, which is when the threads spread it
+            if (MT == 4 || wave < 4) {
+                const uint32_t next = lds_base + (uint32_t)((slot == DS_NS - 1 ? 0 : slot + 1) * S::STAGE);
+                const uint32_t skip_next = skip_a + KBLOCK * (uint32_t)lda;
+                lds_dma16(make_rsrc_words(a + skip_next, a_bytes - skip_next), kb + 1 < kb1 ? voff_a : 0x80000000u,
+                          next + S::PACK_OFF + (uint32_t)(wave * 1024));
+            }
+        } else if (MT == 4 || wave < 4)
             lds_dma16(make_rsrc_words(a + skip_a, a_bytes - skip_a), voff_a, stage + S::MAT_B + (uint32_t)(wave * 1024));
         if (scale_wave == 0)
             lds_dma4(make_rsrc_words(a_scale + (size_t)kb * lda, (uint32_t)lda * 4u), voff_sa, stage + S::SA_OFF);
         else if (scale_wave > 0)
             lds_dma4(make_rsrc_words(b_scale + (size_t)kb * sn, (uint32_t)sn * 4u), voff_sb, stage + S::SB_OFF);
+    };
+    // RAGGED: thread 4 * r + j moves bytes 16 * j .. 16 * j + 15 of packed k-row r (they start at any byte:
+    // five aligned words, shifted) to chunk j of the padded, swizzled row, zeros where the row has ended; only
+    // the chunks of row tiles that exist are written or read.  Reading and writing are apart so that the
+    // stage's matrix work sits between them.
+    const int sp_r = (int)threadIdx.x >> 2, sp_j = (int)threadIdx.x & 3;
+    const bool sp_on = RAGGED && sp_j < mtiles;
+    const uint32_t sp_src = (uint32_t)(S::PACK_OFF + ((sp_r * lda + 16 * sp_j) & ~3));
+    const uint32_t sp_shift = (uint32_t)((sp_r * lda) & 3);
+    const uint32_t sp_dst =
+        (uint32_t)(S::MAT_B + sp_r * S::RSA + ((sp_j ^ (MT == 2 ? (sp_r >> 3) & 1 : (sp_r >> 2) & 3)) << 4));
+    uint32_t sp_mask[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int valid = M - 16 * sp_j - 4 * i;  // bytes of word i inside the row
+        sp_mask[i] = valid >= 4 ? 0xFFFFFFFFu : valid <= 0 ? 0u : (1u << (8 * valid)) - 1u;
+    }
+    uint32_t sp_word[5];
+    auto slab_read = [&](int sl) __attribute__((always_inline)) {
+        if (sp_on) {
+#pragma unroll
+            for (int i = 0; i < 5; ++i)
+                sp_word[i] = *LDS_PTR(uint32_t, lds + sl * S::STAGE + sp_src + 4 * i);
+        }
+    };
+    auto slab_write = [&](int sl) __attribute__((always_inline)) {
+        if (sp_on) {
+            v4i out;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                out[i] = (int)(__builtin_amdgcn_alignbyte(sp_word[i + 1], sp_word[i], sp_shift) & sp_mask[i]);
+            *LDS_PTR(v4i, lds + sl * S::STAGE + sp_dst) = out;
+        }
+    };
+    // wait until at most the copies of `outstanding` stages are in flight (loads complete in order)
+    auto wait_landed = [&](int outstanding) __attribute__((always_inline)) {
+        switch (outstanding) {
+        case 0: ds_wait_vmcnt<0>(); break;
+        case 1: ds_wait_vmcnt<S::COPIES>(); break;
+        case 2: ds_wait_vmcnt<2 * S::COPIES>(); break;
+        case 3: ds_wait_vmcnt<3 * S::COPIES>(); break;
+        case 4: ds_wait_vmcnt<4 * S::COPIES>(); break;
+        default: ds_wait_vmcnt<(DS_NS - 1) * S::COPIES>(); break;
+        }
     };
 
     // ---- transposing reads.  Lane = 16*g + i; read t of a K block covers k-rows 32*t + 8*g + (i >> 1),
@@ -201,41 +264,66 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int nstages = kb1 - kb0;
+    if (RAGGED && (MT == 4 || wave < 4)) {  // the first K block's slab, ahead of every stage
+        const uint32_t skip_a = (uint32_t)kb0 * KBLOCK * (uint32_t)lda;
+        lds_dma16(make_rsrc_words(a + skip_a, a_bytes - skip_a), voff_a, lds_base + S::PACK_OFF + (uint32_t)(wave * 1024));
+    }
 #pragma unroll
     for (int p = 0; p < DS_NS - 1; ++p)
         if (p < nstages)
             issue_stage(p, kb0 + p);
+    if (RAGGED) {  // the first slab has landed once only the stages' copies are in flight
+        wait_landed(nstages < DS_NS - 1 ? nstages : DS_NS - 1);
+        __syncthreads();
+        slab_read(0);
+        slab_write(0);
+    }
     int slot = 0;
     for (int s = 0; s < nstages; ++s) {
         // loads complete in order: this wave's copies of stage s have landed once at most those of the
         // younger stages in flight are outstanding
-        const int younger = nstages - 1 - s < DS_NS - 2 ? nstages - 1 - s : DS_NS - 2;
-        switch (younger) {
-        case 0: ds_wait_vmcnt<0>(); break;
-        case 1: ds_wait_vmcnt<S::COPIES>(); break;
-        case 2: ds_wait_vmcnt<2 * S::COPIES>(); break;
-        case 3: ds_wait_vmcnt<3 * S::COPIES>(); break;
-        default: ds_wait_vmcnt<4 * S::COPIES>(); break;
-        }
-        __syncthreads();  // everyone's copies of stage s landed; the slot of stage s - 1 is no longer read
+        wait_landed(nstages - 1 - s < DS_NS - 2 ? nstages - 1 - s : DS_NS - 2);
+        __syncthreads();  // everyone's copies landed and spreads are done; the slot of stage s - 1 is no longer read
         if (s + DS_NS - 1 < nstages)
             issue_stage(slot == 0 ? DS_NS - 1 : slot - 1, kb0 + s + DS_NS - 1);
         const uint32_t so = (uint32_t)(slot * S::STAGE);
+        const int next_slot = slot == DS_NS - 1 ? 0 : slot + 1;
+        if (RAGGED && s + 1 < nstages)
+            slab_read(next_slot);
         const v8i fb = read_frag(so + addr_b, 32 * 128);
         const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
+        auto multiply = [&](int i, const v8i& fa, float sa) __attribute__((always_inline)) {
+            const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0,
+                                                                             0, 0, 0);
+            const float sc = sa * sb;
+            acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]), fmaf(sc, blk[2], acc[i][2]),
+                           fmaf(sc, blk[3], acc[i][3])};
+        };
+        if (RAGGED) {
+            // every read of this stage is on its way before the spread words are written: the LDS works in order,
+            // and a write between the reads would hold the later ones back by the latency of the slab's words
+            v8i fa[MT];
+            float sa[MT];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            if (i < mtiles) {
-                const v8i fa = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
-                const float sa = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
-                const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    fb, fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                const float sc = sa * sb;
-                acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]),
-                               fmaf(sc, blk[2], acc[i][2]), fmaf(sc, blk[3], acc[i][3])};
-            }
+            for (int i = 0; i < MT; ++i)
+                if (i < mtiles) {
+                    fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
+                    sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
+                }
+            if (s + 1 < nstages)
+                slab_write(next_slot);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                if (i < mtiles)
+                    multiply(i, fa[i], sa[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                if (i < mtiles)
+                    multiply(i, read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA),
+                             *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4));
         }
-        slot = slot == DS_NS - 1 ? 0 : slot + 1;
+        slot = next_slot;
     }
 
     // ---- a lane holds C[16*i + (lane & 15)][n0 + 16*wave + 4*(lane >> 4) + 0..3]
@@ -335,22 +423,22 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     store_c(sum);
 }
 
-template <int MT, int DS_NS>
+template <int MT, int DS_NS, bool RAGGED>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int N, int K,
                     int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
-    decode_body<MT, false, DS_NS>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
+    decode_body<MT, false, DS_NS, RAGGED>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
 }
 
-template <int MT, int DS_NS>
+template <int MT, int DS_NS, bool RAGGED>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
-    decode_body<MT, true, DS_NS>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
+    decode_body<MT, true, DS_NS, RAGGED>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
 }
 
 // The streaming form, for a single problem without a K split whose strips outnumber the workgroups the
@@ -540,9 +628,10 @@ inline bool shallow_ring_pays(long workgroups, int kb_per_split) { return workgr
 
 }  // namespace
 
+// any 1 <= m <= 64: a row count off the 16-byte grid runs the kernels that spread A's packed slabs in the LDS
 bool decode_strip_supports(const GemmArgs& g)
 {
-    return g.m <= 64 && g.m % 16 == 0 && g.n % 16 == 0 && (g.lda == 0 || g.lda == g.m) &&
+    return g.m >= 1 && g.m <= 64 && g.n % 16 == 0 && (g.lda == 0 || g.lda == g.m) &&
            (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) && (reinterpret_cast<uintptr_t>(g.b) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.a_scale) % 4 == 0) && (reinterpret_cast<uintptr_t>(g.b_scale) % 4 == 0) &&
            (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
@@ -622,7 +711,7 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
                            g.k, strips, ksplit, kb_per_split);
         return hipGetLastError();
     };
-    if (ksplit == 1 && strips > STREAM_WORKGROUPS) {  // more units than resident workgroups: one copy stream per workgroup
+    if (ksplit == 1 && strips > STREAM_WORKGROUPS && g.m % 16 == 0) {  // more units than resident workgroups: one copy stream per workgroup
         auto stream = [&](auto kern, int lds) -> hipError_t {
             FP8GEMM_ALLOW_LDS(kern, lds);
             hipLaunchKernelGGL(kern, dim3(STREAM_WORKGROUPS), dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
@@ -632,14 +721,19 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
         return row_tiles(g.m) == 2 ? stream(decode_stream_kernel<2, STREAM_NS>, DecodeShape<2, STREAM_NS>::LDS)
                                    : stream(decode_stream_kernel<4, STREAM_NS>, DecodeShape<4, STREAM_NS>::LDS);
     }
+    if (g.m % 16 != 0)
+        return row_tiles(g.m) == 2 ? go(decode_strip_kernel<2, 6, true>, DecodeShape<2, 6, true>::LDS)
+                                   : go(decode_strip_kernel<4, RAGGED4_NS, true>, DecodeShape<4, RAGGED4_NS, true>::LDS);
     const bool deep = !shallow_ring_pays((long)strips * ksplit, kb_per_split);
     if (row_tiles(g.m) == 2)
-        return deep ? go(decode_strip_kernel<2, 6>, DecodeShape<2, 6>::LDS) : go(decode_strip_kernel<2, 3>, DecodeShape<2, 3>::LDS);
-    return deep ? go(decode_strip_kernel<4, 6>, DecodeShape<4, 6>::LDS) : go(decode_strip_kernel<4, 3>, DecodeShape<4, 3>::LDS);
+        return deep ? go(decode_strip_kernel<2, 6, false>, DecodeShape<2, 6>::LDS)
+                    : go(decode_strip_kernel<2, 3, false>, DecodeShape<2, 3>::LDS);
+    return deep ? go(decode_strip_kernel<4, 6, false>, DecodeShape<4, 6>::LDS)
+                : go(decode_strip_kernel<4, 3, false>, DecodeShape<4, 3>::LDS);
 }
 
-// every group: 1 <= m <= lda <= 64 with lda a multiple of 16 (rows m .. lda-1 of a and a_scale hold zeros),
-// operands aligned like a single problem's
+// every group: 1 <= m <= lda <= 64 (rows m .. lda-1 of a and a_scale readable), operands aligned like a
+// single problem's; one lda off the 16-byte grid sends the whole launch to the slab-spreading kernels
 bool decode_grouped_supports(const GroupTable& tab, int n, int k)
 {
     if (tab.groups < 1 || tab.groups > GroupTable::MAX_GROUPS || k % KBLOCK != 0)
@@ -699,20 +793,27 @@ hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit
     if ((ksplit - 1) * kb_per_split >= nkb)
         return hipErrorInvalidValue;
     int mmax = 0;
-    for (int g = 0; g < tab.groups; ++g)
+    bool ragged = false;
+    for (int g = 0; g < tab.groups; ++g) {
         mmax = tab.lda[g] > mmax ? tab.lda[g] : mmax;
+        ragged |= tab.lda[g] % 16 != 0;
+    }
     const dim3 grid((unsigned)(8 * ((units + 7) / 8) * ksplit));
     auto go = [&](auto kern, int lds) -> hipError_t {
         FP8GEMM_ALLOW_LDS(kern, lds);
         hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), lds, s, tab, mailbox, n, k, strips, ksplit, kb_per_split);
         return hipGetLastError();
     };
+    if (ragged)
+        return row_tiles(mmax) == 2
+                   ? go(decode_strip_grouped_kernel<2, 6, true>, DecodeShape<2, 6, true>::LDS)
+                   : go(decode_strip_grouped_kernel<4, RAGGED4_NS, true>, DecodeShape<4, RAGGED4_NS, true>::LDS);
     const bool deep = !shallow_ring_pays(units * ksplit, kb_per_split);
     if (row_tiles(mmax) == 2)
-        return deep ? go(decode_strip_grouped_kernel<2, 6>, DecodeShape<2, 6>::LDS)
-                    : go(decode_strip_grouped_kernel<2, 3>, DecodeShape<2, 3>::LDS);
-    return deep ? go(decode_strip_grouped_kernel<4, 6>, DecodeShape<4, 6>::LDS)
-                : go(decode_strip_grouped_kernel<4, 3>, DecodeShape<4, 3>::LDS);
+        return deep ? go(decode_strip_grouped_kernel<2, 6, false>, DecodeShape<2, 6>::LDS)
+                    : go(decode_strip_grouped_kernel<2, 3, false>, DecodeShape<2, 3>::LDS);
+    return deep ? go(decode_strip_grouped_kernel<4, 6, false>, DecodeShape<4, 6>::LDS)
+                : go(decode_strip_grouped_kernel<4, 3, false>, DecodeShape<4, 3>::LDS);
 }
 
 }  // namespace fp8gemm

@@ -70,7 +70,9 @@ extern "C" {
  * m % 16 == 0, n % 16 == 0 and 16-byte aligned a, b, a_scale, c as they are; for anything else
  * the library copies the operands concerned into zero-padded buffers in its workspace, runs
  * there and copies c's m x n corner out (plans named "padded_...": one extra launch for the copies and
- * one for c's corner, about 2 bytes of extra traffic per operand byte).  The reference requires M, N % 64 (32) == 0
+ * one for c's corner, about 2 bytes of extra traffic per operand byte).  The decode kernel ("decode128_kN",
+ * chosen for m <= 32) takes any m as it is: a decode batch of 1 ... 15 rows needs no copy.  The reference
+ * requires M, N % 64 (32) == 0
  * and reads out of bounds otherwise (mn_large.hip:16). */
 int fp8_block_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                    void* c, int m, int n, int k);
@@ -130,7 +132,9 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * launch per operand kind ("padded_..._groupedN").  Groups of at most 64 rows (the experts of an MoE
  * layer in a decode step) do not go through 128-row tiles: they run as ONE launch of the decode kernel
  * ("decode128_kN_groupedG": 128-column strips of every group in one work list, every group's B read
- * once, the K range split and added inside the kernel as for a single problem); a call that mixes both
+ * once, the K range split and added inside the kernel as for a single problem; row counts off the 16-row
+ * grid as they are where that is faster -- no group above 16 rows, or a launch of at most 256 strips with
+ * at most 24 K blocks -- else on padded copies of A and a_scale); a call that mixes both
  * kinds launches each kernel once.  More groups than FP8GEMM_MAX_GROUPS fall back to one call
  * of fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to
  * what fp8_block_gemm_stream gives for that problem with the same tile shape (decode kernel: with the

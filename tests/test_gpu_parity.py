@@ -260,6 +260,70 @@ def test_decode_strip_kernel(pkg, m, n, k, ksplit):
         assert np.array_equal(got, again), f"run {rep}: not reproducible"
 
 
+# row counts off the 16-byte grid: the kernel copies A's K blocks as the packed slabs they are and spreads them
+# into padded rows in the LDS (no padded copy of A, no extra launch): one to 63 rows, one and two row tiles and
+# the four-row-tile form, split and unsplit, a ragged last strip, a single K block, more K blocks than ring slots
+DECODE_RAGGED_CASES = [(1, 7168, 2048, 4), (7, 7168, 2048, 4), (8, 7168, 2048, 1), (3, 576, 1024, 3),
+                       (13, 1040, 2048, 16), (2, 96, 512, 2), (5, 128, 128, 1), (31, 4608, 7168, 7),
+                       (17, 1536, 1536, 12), (15, 2048, 384, 3), (24, 16384, 1024, 4), (9, 16, 2048, 1),
+                       (33, 7168, 2048, 4), (47, 1536, 1536, 3), (63, 2064, 7168, 8), (50, 256, 128, 1),
+                       (4, 33040, 384, 1), (36, 512, 3584, 1)]
+
+
+@pytest.mark.parametrize("m,n,k,ksplit", DECODE_RAGGED_CASES)
+def test_decode_strip_kernel_with_rows_off_the_grid(pkg, m, n, k, ksplit):
+    import torch
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1250 + m + n + k + ksplit, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ksplit)
+    assert name == f"decode128_k{ksplit}", name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    # bit-identical to the same problem on zero-padded copies with rows on the grid, and nothing written past row m
+    m16 = (m + 15) // 16 * 16
+    ap = np.zeros((k, m16), np.uint8)
+    ap[:, :m] = a.reshape(k, m)
+    sap = np.zeros((k // 128, m16), np.float32)
+    sap[:, :m] = sa.reshape(k // 128, m)
+    padded, pname = _run(pkg, ap.reshape(-1), b, sap.reshape(-1), sb, m16, n, k, kernel=pkg.KERNEL_SKINNY, variant=1,
+                         ksplit=ksplit)
+    assert pname == name
+    assert np.array_equal(got.reshape(m, n), padded.reshape(m16, n)[:m]), "differs from the padded problem"
+    da, db, dsa, dsb = _dev(a, b, sa, sb)
+    dc = torch.full((m16 + 16, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)
+    pkg.select(pkg.KERNEL_SKINNY)
+    pkg.force_config(1, ksplit)
+    try:
+        pkg.gemm(da, db, dsa, dsb, dc, m, n, k, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+    finally:
+        pkg.select(0)
+        pkg.force_config(-1, 0)
+    out = dc.cpu().numpy().view(np.uint16)
+    assert np.array_equal(out[:m].reshape(-1), got.reshape(-1))
+    assert (out[m:] == 0x7FC1).all(), "rows past m were written"
+
+
+def test_decode_rows_off_the_grid_run_without_a_padded_copy(pkg):
+    """automatic dispatch: a decode batch of seven rows takes the decode kernel directly; with A off a 16-byte
+    boundary it takes the padded plan as before"""
+    import torch
+    m, n, k = 7, 7168, 2048
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1288, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k)
+    assert name.startswith("decode128_k"), name
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    da, db, dsa, dsb = _dev(a, b, sa, sb)
+    shifted = torch.zeros(a.size + 16, dtype=torch.uint8, device="cuda")
+    shifted[4:4 + a.size] = da.view(torch.uint8).reshape(-1)
+    dc = torch.full((m, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16)
+    pkg.gemm(shifted[4:4 + a.size], db, dsa, dsb, dc, m, n, k, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert pkg.last_kernel().startswith("padded_decode128_k"), pkg.last_kernel()
+    assert np.array_equal(dc.cpu().numpy().view(np.uint16).reshape(-1), got.reshape(-1))
+
+
 def test_decode_strip_split_that_outgrows_the_mailbox_is_refused(pkg):
     """128 strips x 15 sending splits x 16 KiB of patches do not fit the 16 MiB mailbox: no such plan"""
     m, n, k = 32, 16384, 2048
@@ -742,7 +806,9 @@ def test_grouped_gemm_pads_groups_off_the_16_byte_grid(pkg, ms, n, k):
     name = pkg.last_kernel()
     # groups of at most 64 rows go to the decode kernel, taller ones to the tile kernel: one launch of each
     parts = name.split("+")
-    assert any(p.startswith("padded_") for p in parts), name           # each launch pads only if its own groups need it
+    # each launch pads only if its own groups need it: the decode kernel takes any row count, the tile kernel
+    # and both kernels' columns need multiples of 16
+    assert any(p.startswith("padded_") for p in parts) == (n % 16 != 0 or any(m > 64 and m % 16 for m in ms)), name
     assert sum(int(p.rsplit("_grouped", 1)[1]) for p in parts) == sum(1 for m in ms if m), name
     assert ("decode128" in name) == any(0 < m <= 64 for m in ms) and ("tile" in name) == any(m > 64 for m in ms), name
     for g, m in enumerate(ms):
@@ -803,11 +869,16 @@ def test_grouped_decode_groups_equal_the_problems_one_by_one(pkg, ms, n, k):
 
 
 def test_grouped_decode_groups_off_the_16_byte_grid_and_mixed_with_tall_groups(pkg):
-    """ragged token counts of 1 to 64 rows run on padded copies in one decode launch; a call that also holds
-    taller groups launches the tile kernel for those; rows beyond m stay untouched"""
+    """ragged token counts of 1 to 64 rows run in one decode launch (on padded copies when n is off the grid, or
+    when that measured faster: groups of more than 16 rows in a launch of more than one round of workgroups or
+    with more than 24 K blocks); a
+    call that also holds taller groups launches the tile kernel for those; rows beyond m stay untouched"""
     import torch
     st = torch.cuda.current_stream().cuda_stream
-    for ms, n, k in [([1, 7, 64, 33, 16, 50, 2], 1536, 1024), ([5, 300, 64, 1000, 17], 640, 512), ([3, 9], 200, 256)]:
+    for ms, n, k in [([1, 7, 64, 33, 16, 50, 2], 1536, 1024), ([5, 300, 64, 1000, 17], 640, 512), ([3, 9], 200, 256),
+                     # more than one round of workgroups: rows taken as they are while no group has more than 16,
+                     # padded copies of A beyond (faster there)
+                     ([3, 16, 9, 1] * 6, 2048, 384), ([17, 31, 5, 20] * 5, 2048, 384), ([20, 7], 256, 3328)]:
         host, dev, outs = [], [], []
         for g, m in enumerate(ms):
             a, b, sa, sb = oracle.make_inputs(m, n, k, 9300 + 11 * g + n)
@@ -819,7 +890,9 @@ def test_grouped_decode_groups_off_the_16_byte_grid_and_mixed_with_tall_groups(p
                          outs, ms, n, k, st)
         torch.cuda.synchronize()
         name = pkg.last_kernel()
-        assert "decode128_k" in name and name.startswith("padded_"), name
+        small = [m for m in ms if m <= 64]
+        as_they_are = max(small) <= 16 or (len(small) * -(-n // 128) <= 256 and k <= 24 * 128)
+        assert "decode128_k" in name and name.startswith("padded_decode128_k") == (n % 16 != 0 or not as_they_are), name
         if max(ms) > 64:
             assert "+" in name and "tile" in name, name
         for g, m in enumerate(ms):
