@@ -106,7 +106,10 @@ struct DecodeProblem {
 // Work units = (problem, strip), numbered problem-major; `units` of them.  Linear workgroup ids that
 // agree modulo 8 share an XCD: the ksplit workgroups of unit u sit at ids xcd + 8 * (grp * ksplit + split)
 // with u = grp * 8 + xcd.
-template <int MT, bool GROUPED, int DS_NS, bool RAGGED>
+// TILES = the number of 16-row tiles when the launch knows it (a single problem), 0 = read from the problem (grouped
+// launches): with the count fixed the K loop has no branch around its LDS operations, and the compiler's wait
+// counts name exactly the reads an MFMA needs (around a branch it waits for everything in flight).
+template <int MT, bool GROUPED, int DS_NS, bool RAGGED, int TILES>
 __device__ __forceinline__ void decode_body(const DecodeProblem& one, const GroupTable* tab, float* mailbox, int N, int K,
                                             int strips, int units, int ksplit, int kb_per_split)
 {
@@ -143,7 +146,7 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     const int kb0 = split * kb_per_split;
     const int kb1 = (kb0 + kb_per_split < nkb) ? (kb0 + kb_per_split) : nkb;
     const int sn = (N + KBLOCK - 1) / KBLOCK;
-    const int mtiles = (M + 15) >> 4;  // 1 .. MT
+    const int mtiles = TILES > 0 ? TILES : (M + 15) >> 4;  // 1 .. MT
 
     // ---- copy plan.  B: instruction q (0, 1) of a wave fills stage rows 16*wave + 8*q + (lane >> 3), chunk
     // position lane & 7; the chunk swizzle (r >> 1) & 7 is (4*q + (lane >> 4)) & 7.  A, 32-byte rows: waves
@@ -199,14 +202,17 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     };
     // RAGGED: thread 4 * r + j moves bytes 16 * j .. 16 * j + 15 of packed k-row r (they start at any byte:
     // five aligned words, shifted) to chunk j of the padded, swizzled row, zeros where the row has ended; only
-    // the chunks of row tiles that exist are written or read.  Reading and writing are apart so that the
-    // stage's matrix work sits between them.
+    // the chunks of row tiles that exist are read by the MFMAs.  Every thread reads and writes, so that no branch
+    // surrounds the LDS operations: a thread whose chunk belongs to no row tile reads what lies at its address
+    // (inside the stage) and writes to the 16 spare bytes behind the slab.  Reading and writing are apart so that
+    // the stage's other LDS reads sit between them.
     const int sp_r = (int)threadIdx.x >> 2, sp_j = (int)threadIdx.x & 3;
-    const bool sp_on = RAGGED && sp_j < mtiles;
     const uint32_t sp_src = (uint32_t)(S::PACK_OFF + ((sp_r * lda + 16 * sp_j) & ~3));
     const uint32_t sp_shift = (uint32_t)((sp_r * lda) & 3);
     const uint32_t sp_dst =
-        (uint32_t)(S::MAT_B + sp_r * S::RSA + ((sp_j ^ (MT == 2 ? (sp_r >> 3) & 1 : (sp_r >> 2) & 3)) << 4));
+        sp_j < mtiles
+            ? (uint32_t)(S::MAT_B + sp_r * S::RSA + ((sp_j ^ (MT == 2 ? (sp_r >> 3) & 1 : (sp_r >> 2) & 3)) << 4))
+            : (uint32_t)(S::PACK_OFF + S::MAT_A);
     uint32_t sp_mask[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -215,20 +221,16 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     }
     uint32_t sp_word[5];
     auto slab_read = [&](int sl) __attribute__((always_inline)) {
-        if (sp_on) {
 #pragma unroll
-            for (int i = 0; i < 5; ++i)
-                sp_word[i] = *LDS_PTR(uint32_t, lds + sl * S::STAGE + sp_src + 4 * i);
-        }
+        for (int i = 0; i < 5; ++i)
+            sp_word[i] = *LDS_PTR(uint32_t, lds + sl * S::STAGE + sp_src + 4 * i);
     };
     auto slab_write = [&](int sl) __attribute__((always_inline)) {
-        if (sp_on) {
-            v4i out;
+        v4i out;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                out[i] = (int)(__builtin_amdgcn_alignbyte(sp_word[i + 1], sp_word[i], sp_shift) & sp_mask[i]);
-            *LDS_PTR(v4i, lds + sl * S::STAGE + sp_dst) = out;
-        }
+        for (int i = 0; i < 4; ++i)
+            out[i] = (int)(__builtin_amdgcn_alignbyte(sp_word[i + 1], sp_word[i], sp_shift) & sp_mask[i]);
+        *LDS_PTR(v4i, lds + sl * S::STAGE + sp_dst) = out;
     };
     // wait until at most the copies of `outstanding` stages are in flight (loads complete in order)
     auto wait_landed = [&](int outstanding) __attribute__((always_inline)) {
@@ -288,7 +290,8 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
             issue_stage(slot == 0 ? DS_NS - 1 : slot - 1, kb0 + s + DS_NS - 1);
         const uint32_t so = (uint32_t)(slot * S::STAGE);
         const int next_slot = slot == DS_NS - 1 ? 0 : slot + 1;
-        if (RAGGED && s + 1 < nstages)
+        // RAGGED: the next stage's slab, also behind the last stage (nothing reads what that spreads)
+        if (RAGGED)
             slab_read(next_slot);
         const v8i fb = read_frag(so + addr_b, 32 * 128);
         const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
@@ -299,24 +302,24 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
             acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]), fmaf(sc, blk[2], acc[i][2]),
                            fmaf(sc, blk[3], acc[i][3])};
         };
-        if (RAGGED) {
-            // every read of this stage is on its way before the spread words are written: the LDS works in order,
-            // and a write between the reads would hold the later ones back by the latency of the slab's words
-            v8i fa[MT];
-            float sa[MT];
+        if (TILES > 0) {
+            // every read of the stage is on its way before the first MFMA (and before the spread words are
+            // written: the LDS works in order, a write among the reads would hold the later ones back)
+            v8i fa[TILES > 0 ? TILES : 1];
+            float sa[TILES > 0 ? TILES : 1];
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
-                if (i < mtiles) {
-                    fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
-                    sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
-                }
-            if (s + 1 < nstages)
+            for (int i = 0; i < TILES; ++i) {
+                sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
+                fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
+            }
+            if (RAGGED)
                 slab_write(next_slot);
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
-                if (i < mtiles)
-                    multiply(i, fa[i], sa[i]);
+            for (int i = 0; i < TILES; ++i)
+                multiply(i, fa[i], sa[i]);
         } else {
+            if (RAGGED)
+                slab_write(next_slot);
 #pragma unroll
             for (int i = 0; i < MT; ++i)
                 if (i < mtiles)
@@ -423,14 +426,14 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     store_c(sum);
 }
 
-template <int MT, int DS_NS, bool RAGGED>
+template <int MT, int DS_NS, bool RAGGED, int TILES>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int N, int K,
                     int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
-    decode_body<MT, false, DS_NS, RAGGED>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
+    decode_body<MT, false, DS_NS, RAGGED, TILES>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
 }
 
 template <int MT, int DS_NS, bool RAGGED>
@@ -438,7 +441,7 @@ __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
-    decode_body<MT, true, DS_NS, RAGGED>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
+    decode_body<MT, true, DS_NS, RAGGED, 0>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
 }
 
 // The streaming form, for a single problem without a K split whose strips outnumber the workgroups the
@@ -721,15 +724,25 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
         return row_tiles(g.m) == 2 ? stream(decode_stream_kernel<2, STREAM_NS>, DecodeShape<2, STREAM_NS>::LDS)
                                    : stream(decode_stream_kernel<4, STREAM_NS>, DecodeShape<4, STREAM_NS>::LDS);
     }
-    if (g.m % 16 != 0)
-        return row_tiles(g.m) == 2 ? go(decode_strip_kernel<2, 6, true>, DecodeShape<2, 6, true>::LDS)
-                                   : go(decode_strip_kernel<4, RAGGED4_NS, true>, DecodeShape<4, RAGGED4_NS, true>::LDS);
+    const int tiles = (g.m + 15) / 16;
+    if (g.m % 16 != 0) {
+        constexpr int L2 = DecodeShape<2, 6, true>::LDS, L4 = DecodeShape<4, RAGGED4_NS, true>::LDS;
+        switch (tiles) {
+        case 1: return go(decode_strip_kernel<2, 6, true, 1>, L2);
+        case 2: return go(decode_strip_kernel<2, 6, true, 2>, L2);
+        case 3: return go(decode_strip_kernel<4, RAGGED4_NS, true, 3>, L4);
+        default: return go(decode_strip_kernel<4, RAGGED4_NS, true, 4>, L4);
+        }
+    }
     const bool deep = !shallow_ring_pays((long)strips * ksplit, kb_per_split);
-    if (row_tiles(g.m) == 2)
-        return deep ? go(decode_strip_kernel<2, 6, false>, DecodeShape<2, 6>::LDS)
-                    : go(decode_strip_kernel<2, 3, false>, DecodeShape<2, 3>::LDS);
-    return deep ? go(decode_strip_kernel<4, 6, false>, DecodeShape<4, 6>::LDS)
-                : go(decode_strip_kernel<4, 3, false>, DecodeShape<4, 3>::LDS);
+    constexpr int D2 = DecodeShape<2, 6>::LDS, S2 = DecodeShape<2, 3>::LDS, D4 = DecodeShape<4, 6>::LDS,
+                  S4 = DecodeShape<4, 3>::LDS;
+    switch (tiles) {
+    case 1: return deep ? go(decode_strip_kernel<2, 6, false, 1>, D2) : go(decode_strip_kernel<2, 3, false, 1>, S2);
+    case 2: return deep ? go(decode_strip_kernel<2, 6, false, 2>, D2) : go(decode_strip_kernel<2, 3, false, 2>, S2);
+    case 3: return deep ? go(decode_strip_kernel<4, 6, false, 3>, D4) : go(decode_strip_kernel<4, 3, false, 3>, S4);
+    default: return deep ? go(decode_strip_kernel<4, 6, false, 4>, D4) : go(decode_strip_kernel<4, 3, false, 4>, S4);
+    }
 }
 
 // every group: 1 <= m <= lda <= 64 (rows m .. lda-1 of a and a_scale readable), operands aligned like a
