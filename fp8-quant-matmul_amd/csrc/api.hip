@@ -740,18 +740,11 @@ int run_grouped_table(const GroupTable& tab, int n, int k, bool decode, hipStrea
     const size_t nkb = (size_t)k / 128;
     bool pad_a = false, pad_b = n16 != n, pad_c = n16 != n;
     // The decode kernel takes row counts off the 16-byte grid as they are (it spreads A's packed slabs in the
-    // LDS, which costs it 0.1 us per K block and workgroup) and 4-byte aligned scales.  Measured on 2 to 64 groups,
-    // N = 1536 ... 7168, K = 2048 and 7168 against the padded copies (one more launch, 2 - 4 us, then the plain
-    // kernel): 10 - 30 % faster while no group has more than 16 rows, or the launch is one round of workgroups
-    // with at most 24 K blocks; 3 - 12 % slower beyond.
-    int mmax = 0;
-    for (int g = 0; g < tab.groups; ++g)
-        mmax = tab.m[g] > mmax ? tab.m[g] : mmax;
-    const bool spread_pays =
-        decode && (mmax <= 16 || ((long)tab.groups * ((n16 + 127) / 128) <= NUM_CU && nkb <= 24));
+    // LDS) and 4-byte aligned scales: measured on 2 to 64 groups of 1 - 64 rows, N = 1536 ... 7168, K = 2048 and
+    // 7168, level with the padded copies (one more launch, then the plain kernel) or up to 20 % ahead.
     for (int g = 0; g < tab.groups; ++g) {
-        pad_a = pad_a || misaligned16(tab.a[g]) || (tab.m[g] % 16 != 0 && !spread_pays) ||
-                (!decode && misaligned16(tab.a_scale[g]));
+        pad_a = pad_a || misaligned16(tab.a[g]) ||
+                (!decode && (tab.m[g] % 16 != 0 || misaligned16(tab.a_scale[g])));
         pad_b = pad_b || misaligned16(tab.b[g]);
         pad_c = pad_c || misaligned16(tab.c[g]);
     }

@@ -106,9 +106,8 @@ struct DecodeProblem {
 // Work units = (problem, strip), numbered problem-major; `units` of them.  Linear workgroup ids that
 // agree modulo 8 share an XCD: the ksplit workgroups of unit u sit at ids xcd + 8 * (grp * ksplit + split)
 // with u = grp * 8 + xcd.
-// TILES = the number of 16-row tiles when the launch knows it (a single problem), 0 = read from the problem (grouped
-// launches): with the count fixed the K loop has no branch around its LDS operations, and the compiler's wait
-// counts name exactly the reads an MFMA needs (around a branch it waits for everything in flight).
+// TILES = the number of 16-row tiles when the launch knows it (a single problem: the count is then a constant
+// in the epilogue as well), 0 = read from the problem (grouped launches).
 template <int MT, bool GROUPED, int DS_NS, bool RAGGED, int TILES>
 __device__ __forceinline__ void decode_body(const DecodeProblem& one, const GroupTable* tab, float* mailbox, int N, int K,
                                             int strips, int units, int ksplit, int kb_per_split)
@@ -280,6 +279,12 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         slab_read(0);
         slab_write(0);
     }
+    // The K loop, one copy per number of 16-row tiles (chosen below, outside the loop): with the count fixed
+    // the loop has no branch around its LDS operations, every read of a stage is issued before the first MFMA,
+    // and the compiler's wait counts name exactly the reads each MFMA needs (around a branch it waits for
+    // everything in flight, which serialises read latency and MFMAs tile after tile).
+    auto k_loop = [&](auto tile_count) __attribute__((always_inline)) {
+    constexpr int T = decltype(tile_count)::value;
     int slot = 0;
     for (int s = 0; s < nstages; ++s) {
         // loads complete in order: this wave's copies of stage s have landed once at most those of the
@@ -302,31 +307,37 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
             acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]), fmaf(sc, blk[2], acc[i][2]),
                            fmaf(sc, blk[3], acc[i][3])};
         };
-        if (TILES > 0) {
-            // every read of the stage is on its way before the first MFMA (and before the spread words are
-            // written: the LDS works in order, a write among the reads would hold the later ones back)
-            v8i fa[TILES > 0 ? TILES : 1];
-            float sa[TILES > 0 ? TILES : 1];
+        // the spread words are written behind the stage's reads: the LDS works in order, a write among the
+        // reads would hold the later ones back
+        v8i fa[T];
+        float sa[T];
 #pragma unroll
-            for (int i = 0; i < TILES; ++i) {
-                sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
-                fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
-            }
-            if (RAGGED)
-                slab_write(next_slot);
-#pragma unroll
-            for (int i = 0; i < TILES; ++i)
-                multiply(i, fa[i], sa[i]);
-        } else {
-            if (RAGGED)
-                slab_write(next_slot);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-                if (i < mtiles)
-                    multiply(i, read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA),
-                             *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4));
+        for (int i = 0; i < T; ++i) {
+            sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
+            fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
         }
+        if (RAGGED)
+            slab_write(next_slot);
+#pragma unroll
+        for (int i = 0; i < T; ++i)
+            multiply(i, fa[i], sa[i]);
         slot = next_slot;
+    }
+    };
+    if (TILES > 0)
+        k_loop(std::integral_constant<int, (TILES > 0 ? TILES : 1)>{});
+    else
+    switch (mtiles) {
+    case 1: k_loop(std::integral_constant<int, 1>{}); break;
+    case 2: k_loop(std::integral_constant<int, 2>{}); break;
+    case 3:
+        if (MT == 4)
+            k_loop(std::integral_constant<int, MT == 4 ? 3 : 1>{});
+        break;
+    default:
+        if (MT == 4)
+            k_loop(std::integral_constant<int, MT == 4 ? 4 : 1>{});
+        break;
     }
 
     // ---- a lane holds C[16*i + (lane & 15)][n0 + 16*wave + 4*(lane >> 4) + 0..3]
