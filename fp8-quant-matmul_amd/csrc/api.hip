@@ -168,13 +168,17 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     const double area = (double)bm * bn / 65536.0;
     // (the 256x256 tile measures 3-5 % ahead of 256x192 per flop where both fill their rounds; the fitted
     // line, extrapolated to its area, would put it 6 % ahead)
-    const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0);
+    // (a single row of tiles reads every byte of B once and from HBM -- decode weights do not fit the caches --,
+    // where a K block takes a quarter longer than the fit to cached operands says: without this factor
+    // 48 x 7168 x 1536 stays unsplit, 9.4 us from HBM against 8.1 us with two splits)
+    const double per_kb =
+        (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * (g.m <= 64 ? 1.25 : 1.0);
     const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     const long items = (long)tiles * ksplit;
-    // two 64x64 workgroups share a CU; counted only for a single row of tiles (M <= 64), where the K
-    // split decides everything: the constants above were fitted to taller problems without it
-    const long slots = (variant == TILE_64x64 && g.m <= 64) ? 2 * NUM_CU : NUM_CU;
-    const long rounds = (items + slots - 1) / slots;
+    // (two 64x64 workgroups share a CU, but a single row of tiles with B from HBM is fastest with at most one
+    // workgroup per CU: M = 48, 64 on 12 shapes, the split that keeps tiles x splits within 256 is the best
+    // measured or within 2 % of it)
+    const long rounds = (items + NUM_CU - 1) / NUM_CU;
     double cost = 1.79 + rounds * per_item;
     if (ksplit > 1 && fused)  // the last split of a tile waits for the others' accumulators and reads them
         cost += 1.8 + 0.35 * (ksplit - 1) * (double)(bm * bn) / 4096.0;
@@ -303,7 +307,10 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
         // With more than 32 rows the 64x64 tile plans that add their K splits in the kernel are ahead of the wide
         // strips on 22 of 24 shapes (M = 48, 64; same N and K; from HBM 6.2-15 us against 7.5-16 us): the
         // four-row-tile form is there for grouped launches and runs single problems only when asked for by name.
-        if (!by_name && g.m > 32)
+        // ... except where N x K is large (N = 7168, K >= 4096: 12.2 - 17.4 us against 13.7 - 20.4 us), and for row
+        // counts off the 16-byte grid, which the strips take as they are while the tiles need padded copies
+        // (M = 33 ... 63 on the same 12 shapes: 6.8 - 16.9 us against 10.8 - 23.8 us).
+        if (!by_name && g.m > 32 && g.m % 16 == 0 && !(g.n >= 6144 && (long long)g.n * g.k >= 28000000ll))
             wide_us = 1e300;
         if (!by_name && cfg.force_variant < 0 && cfg.force_ksplit <= 0 && wide_us < 1e300 && cfg.fused_ok)
             return wide;
@@ -382,9 +389,11 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
             const int kbs = (nkb + ks - 1) / ks;
             if ((ks - 1) * kbs >= nkb)
                 continue;
-            // a single row of tiles: the fitted constants overrate a split into short K ranges (measured
-            // for M = 16 ... 64: the best split never leaves a workgroup fewer than 8 K blocks)
-            if (g.m <= 64 && fk <= 0 && selected == FP8GEMM_KERNEL_AUTO && ks > 1 && kbs < 8)
+            // a single row of tiles: the fitted constants overrate a split into short K ranges (measured for
+            // M = 16 ... 64: with the reduction kernel the best split never leaves a workgroup fewer than 8 K
+            // blocks; with the splits added inside the kernel, never fewer than 3)
+            if (g.m <= 64 && fk <= 0 && selected == FP8GEMM_KERNEL_AUTO && ks > 1 &&
+                kbs < (tile_plan_fused(g, v, ks, cfg) ? 3 : 8))
                 continue;
             const double cst = tile_cost(g, v, ks, tile_plan_fused(g, v, ks, cfg));
             if (cst < best) {

@@ -464,7 +464,7 @@ decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, 
 // bit-identical results.  Grouped launches gain nothing from it (64 groups x 56 strips: 225 against 220 us)
 // and keep the plain form.  (A strip's two stores per wave share the vmcnt counter with the copies and may
 // complete after younger copies; counting them as outstanding copies only makes a wait longer, never shorter.)
-template <int MT, int DS_NS>
+template <int MT, int DS_NS, int TILES>
 __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int N, int K, int units)
 {
     using S = DecodeShape<MT, DS_NS>;
@@ -549,7 +549,6 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
     };
     v4f acc[MT];
     const DecodeProblem mp = one;
-    const int mtiles = (mp.M + 15) >> 4;
     int mp_strip = 0;
 
 #pragma unroll
@@ -576,17 +575,21 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
         const uint32_t so = (uint32_t)(slot * S::STAGE);
         const v8i fb = read_frag(so + addr_b, 32 * 128);
         const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
+        // TILES 16-row tiles (fixed per launch): every read of the stage is issued before the first MFMA
+        v8i fa[TILES];
+        float sa[TILES];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            if (i < mtiles) {
-                const v8i fa = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
-                const float sa = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
-                const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    fb, fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                const float sc = sa * sb;
-                acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]),
-                               fmaf(sc, blk[2], acc[i][2]), fmaf(sc, blk[3], acc[i][3])};
-            }
+        for (int i = 0; i < TILES; ++i) {
+            sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
+            fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
+        }
+#pragma unroll
+        for (int i = 0; i < TILES; ++i) {
+            const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[i], (v4f){0.f, 0.f, 0.f, 0.f}, 0,
+                                                                             0, 0, 0, 0, 0);
+            const float sc = sa[i] * sb;
+            acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]), fmaf(sc, blk[2], acc[i][2]),
+                           fmaf(sc, blk[3], acc[i][3])};
         }
         slot = slot == DS_NS - 1 ? 0 : slot + 1;
         if (++kb == nkb) {
@@ -608,13 +611,13 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
     }
 }
 
-template <int MT, int DS_NS>
+template <int MT, int DS_NS, int TILES>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_stream_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
                      const float* __restrict__ b_scale, uint16_t* __restrict__ c, int M, int N, int K, int strips)
 {
     const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
-    decode_stream_body<MT, DS_NS>(one, N, K, strips);
+    decode_stream_body<MT, DS_NS, TILES>(one, N, K, strips);
 }
 
 // records the XCC (XCD) id each workgroup of a probe grid runs on
@@ -671,7 +674,10 @@ double decode_strip_cost(const GemmArgs& g, int ksplit)
     const int nkb = g.k / KBLOCK;
     const int kbs = (nkb + ksplit - 1) / ksplit;
     const long wgs = (long)strips * ksplit;
-    const long rounds = (wgs + 255) / 256;
+    // the splits of a strip share an XCD (32 CUs, one workgroup each), strips are dealt out over the eight XCDs:
+    // 36 strips x 7 splits are 252 workgroups, but 35 on each of four XCDs, which is two rounds there (measured:
+    // 19.8 us against 14.0 us with 6 splits for 4608 x 7168)
+    const long rounds = ((long)((strips + 7) / 8) * ksplit + 31) / 32;
     const double active = wgs < 256 ? (double)wgs : 256.0;
     const double per_block = 0.50 + 0.001 * active;
     const double life = 1.0 + kbs * per_block + (ksplit > 1 ? 0.39 * ksplit : 0.0);
@@ -732,8 +738,12 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
                                g.m, g.n, g.k, strips);
             return hipGetLastError();
         };
-        return row_tiles(g.m) == 2 ? stream(decode_stream_kernel<2, STREAM_NS>, DecodeShape<2, STREAM_NS>::LDS)
-                                   : stream(decode_stream_kernel<4, STREAM_NS>, DecodeShape<4, STREAM_NS>::LDS);
+        switch (g.m / 16) {
+        case 1: return stream(decode_stream_kernel<2, STREAM_NS, 1>, DecodeShape<2, STREAM_NS>::LDS);
+        case 2: return stream(decode_stream_kernel<2, STREAM_NS, 2>, DecodeShape<2, STREAM_NS>::LDS);
+        case 3: return stream(decode_stream_kernel<4, STREAM_NS, 3>, DecodeShape<4, STREAM_NS>::LDS);
+        default: return stream(decode_stream_kernel<4, STREAM_NS, 4>, DecodeShape<4, STREAM_NS>::LDS);
+        }
     }
     const int tiles = (g.m + 15) / 16;
     if (g.m % 16 != 0) {

@@ -225,8 +225,15 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(32, 16384, 7168) == "decode128_k2"     # 128 strips x 2
     assert pkg.plan(32, 128, 128) == "decode128_k1"        # one K block: nothing to split
     assert pkg.workspace_bytes(32, 7168, 2048) == pkg.WORKSPACE_HEADER_BYTES   # the splits meet in the header's mailbox
-    assert pkg.plan(64, 1536, 7168) == "tile64x64_k7f"     # a single row of tiles: never fewer than 8 K blocks per split
-    assert pkg.plan(48, 1536, 1536) == "tile64x64_k1"
+    # 33 ... 64 rows: 64x64 tiles with the K range split inside the kernel, tiles x splits within one workgroup
+    # per CU and at least 3 K blocks per split; the wide strips where N x K is large or the row count is off
+    # the 16-byte grid (the strips take it as it is, the tiles would need padded copies)
+    assert pkg.plan(64, 1536, 7168) == "tile64x64_k8f"     # 24 tiles x 8
+    assert pkg.plan(48, 1536, 1536) == "tile64x64_k4f"     # 3 K blocks per split
+    assert pkg.plan(64, 7168, 2048) == "tile64x64_k2f"     # 112 tiles x 2
+    assert pkg.plan(64, 7168, 7168) == "decode128_k4"
+    assert pkg.plan(40, 4608, 7168) == "decode128_k6"      # 36 strips over 8 XCDs: 5 x 6 workgroups on an XCD's 32 CUs
+    assert pkg.plan(7, 7168, 2048) == "decode128_k4"       # a decode batch of 7 rows: no padded copy
     pkg.select(pkg.KERNEL_SKINNY)
     pkg.force_config(-1, 3)
     assert pkg.plan(32, 7168, 2048) == "decode128_k3"      # a pinned K split reaches the decode kernels too
