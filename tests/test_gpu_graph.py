@@ -32,6 +32,8 @@ CASES = [
     (32, 1024, 512, 0, -1, 0, -1),      # decode shape under automatic dispatch
     (32, 1024, 512, 4, 0, 0, -1),       # narrow-strip decode kernel
     (32, 2048, 2048, 4, 1, 4, -1),      # wide-strip decode kernel, K splits added inside the kernel (mailbox in the workspace header)
+    (5, 2048, 2048, 0, -1, 0, -1),      # a decode batch off the 16-row grid: rows taken as they are, no copy launch in the graph
+    (40, 1536, 1024, 0, -1, 0, -1),     # the same with three row tiles
     (256, 384, 512, 0, -1, 0, -1),      # small tile kernel picked by the dispatcher
     (512, 512, 384, 0, 2, 0, 1),        # persistent form
     (256, 256, 1024, 3, 2, 4, -1),      # K split over workgroups + reduction, caller's workspace
