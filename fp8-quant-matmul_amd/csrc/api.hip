@@ -750,10 +750,12 @@ int run_grouped_table(const GroupTable& tab, int n, int k, bool decode, hipStrea
     bool pad_a = false, pad_b = n16 != n, pad_c = n16 != n;
     // The decode kernel takes row counts off the 16-byte grid as they are (it spreads A's packed slabs in the
     // LDS) and 4-byte aligned scales: measured on 2 to 64 groups of 1 - 64 rows, N = 1536 ... 7168, K = 2048 and
-    // 7168, level with the padded copies (one more launch, then the plain kernel) or up to 20 % ahead.
+    // 7168, level with the padded copies (one more launch, then the plain kernel) or up to 20 % ahead.  Launches
+    // large enough for the streaming form, which wants rows on the grid, are the exception: 9 % for one copy launch.
+    const bool streams = decode && decode_grouped_streams(tab.groups, n16);
     for (int g = 0; g < tab.groups; ++g) {
-        pad_a = pad_a || misaligned16(tab.a[g]) ||
-                (!decode && (tab.m[g] % 16 != 0 || misaligned16(tab.a_scale[g])));
+        pad_a = pad_a || misaligned16(tab.a[g]) || (tab.m[g] % 16 != 0 && (!decode || streams)) ||
+                (!decode && misaligned16(tab.a_scale[g]));
         pad_b = pad_b || misaligned16(tab.b[g]);
         pad_c = pad_c || misaligned16(tab.c[g]);
     }

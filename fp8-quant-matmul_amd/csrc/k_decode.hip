@@ -66,13 +66,17 @@ constexpr unsigned long long SPIN_LIMIT_TICKS = 100000000ull;  // one second of 
 // RAGGED = the row count is not a multiple of 16, so that k-rows of A do not start on 16-byte boundaries: a stage
 // then also holds the K block's slab of A as it lies in memory, [128][M] bytes packed -- which does start on a
 // 16-byte boundary, 128 * M * kb bytes into A -- and the threads spread it into the padded rows the reads expect.
-template <int MT, int DS_NS, bool RAGGED = false>
+// NB = 128-column halves of a strip (1; 2 in the streaming form of wide problems: 256 contiguous bytes of every
+// k-row instead of 128, which the memory system serves 10 % faster, and A's fragments used twice).  Each half is a
+// [128][128] byte matrix of its own in the stage, laid out and swizzled alike.
+template <int MT, int DS_NS, bool RAGGED = false, int NB = 1>
 struct DecodeShape {
     static constexpr int RSA = 16 * MT;                 // LDS bytes per k-row of A
-    static constexpr int MAT_B = KBLOCK * 128;
+    static constexpr int HALF_B = KBLOCK * 128;
+    static constexpr int MAT_B = HALF_B * NB;
     static constexpr int MAT_A = KBLOCK * RSA;
     static constexpr int SA_OFF = MAT_B + MAT_A;        // up to 64 a_scale floats
-    static constexpr int SB_OFF = SA_OFF + 256;         // 1 float (every wave that brings it writes the same bytes)
+    static constexpr int SB_OFF = SA_OFF + 256;         // NB floats (every wave that brings them writes the same bytes)
     static constexpr int PACK_OFF = SB_OFF + 256;       // RAGGED: the packed slab of A, up to MAT_A bytes, and 16
     // bytes the last row's reads may run into; stages start on 512-byte boundaries
     static constexpr int STAGE = RAGGED ? (PACK_OFF + MAT_A + 16 + 511) / 512 * 512 : PACK_OFF;
@@ -80,7 +84,7 @@ struct DecodeShape {
     // copy instructions per wave and stage: two of B, then A / scales
     //   MT = 2: waves 0..3 A (32 rows x 32 B each), wave 4 a_scale, waves 5..7 b_scale
     //   MT = 4: every wave A (16 rows x 64 B each), then wave 0 a_scale, waves 1..7 b_scale
-    static constexpr int COPIES = MT == 2 ? 3 : 4;
+    static constexpr int COPIES = 2 * NB + (MT == 2 ? 1 : 2);
     static_assert(MT == 2 || MT == 4, "two or four row tiles");
     static_assert(LDS <= 160 * 1024, "ring exceeds the LDS");
     static_assert(COPIES * (DS_NS - 1) < 64, "vmcnt is a 6-bit field");
@@ -464,10 +468,19 @@ decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, 
 // bit-identical results.  Grouped launches gain nothing from it (64 groups x 56 strips: 225 against 220 us)
 // and keep the plain form.  (A strip's two stores per wave share the vmcnt counter with the copies and may
 // complete after younger copies; counting them as outstanding copies only makes a wait longer, never shorter.)
-template <int MT, int DS_NS, int TILES>
-__device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int N, int K, int units)
+// STAGED: a strip's C goes through the LDS (behind the ring) and leaves in whole rows, 16 bytes per lane, instead
+// of 32 bytes of a row per wave straight from the accumulators (3 - 10 % on four row tiles, nothing on two: what
+// C costs a long stream -- 15 % of the run time for 3 % of the bytes at 32 rows and K = 2048 -- is the price of
+// writes to HBM among the reads, whatever their shape).  Needs c on a 16-byte boundary.
+// GROUPED: units run through the strips of all problems of `tab` (TILES = 0: the tile count is the unit's own, and
+// the stage's math is chosen by it -- one straight-line copy per count).
+template <int MT, int DS_NS, int TILES, bool STAGED, int NB, bool GROUPED>
+__device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, const GroupTable* tab, int N, int K, int strips,
+                                                   int units)
 {
-    using S = DecodeShape<MT, DS_NS>;
+    using S = DecodeShape<MT, DS_NS, false, NB>;
+    constexpr int BN = DS_BN * NB;                 // columns of a strip
+    constexpr int C_STAGE_ROW = 2 * BN + 16;       // bytes per staged row of C (16 more than the data: rows 4 banks apart)
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     auto lds = LDS_PTR(uint8_t, smem);
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -480,21 +493,33 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
     const int sn = (N + KBLOCK - 1) / KBLOCK;
     const int total = ((units - w + G - 1) / G) * nkb;  // stages of this workgroup's stream
 
+    auto problem_of = [&](int unit, int* strip) __attribute__((always_inline)) -> DecodeProblem {
+        if (!GROUPED) {
+            *strip = unit;
+            return one;
+        }
+        const int g = unit / strips;
+        *strip = unit - g * strips;
+        return DecodeProblem{tab->a[g], tab->b[g], tab->a_scale[g], tab->b_scale[g], tab->c[g], tab->m[g], tab->lda[g]};
+    };
     // ---- copy side: what the strip being copied needs (see decode_body for the plan)
-    const DecodeProblem cp = one;
+    DecodeProblem cp = one;
     int cp_strip = 0;
-    uint32_t voff_b[2] = {0, 0}, voff_a = 0, voff_sa = 0, voff_sb = 0;
+    uint32_t voff_b[NB][2], voff_a = 0, voff_sa = 0, voff_sb = 0;
     auto enter_copy_unit = [&](int unit) __attribute__((always_inline)) {
-        cp_strip = unit;
-        const int n0 = cp_strip * DS_BN;
+        cp = problem_of(unit, &cp_strip);
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const int cc = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
-            const bool ok = n0 + 16 * cc < N;
-            voff_b[q] = ok ? (uint32_t)((16 * wave + 8 * q + (lane >> 3)) * N + n0 + 16 * cc) : 0x80000000u;
+        for (int h = 0; h < NB; ++h) {
+            const int n0 = cp_strip * BN + DS_BN * h;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int cc = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
+                const bool ok = n0 + 16 * cc < N;
+                voff_b[h][q] = ok ? (uint32_t)((16 * wave + 8 * q + (lane >> 3)) * N + n0 + 16 * cc) : 0x80000000u;
+            }
         }
         voff_sa = lane < cp.lda ? (uint32_t)(lane * 4) : 0x80000000u;
-        voff_sb = lane == 0 ? (uint32_t)(cp_strip * 4) : 0x80000000u;
+        voff_sb = lane < NB ? (uint32_t)((cp_strip * NB + lane) * 4) : 0x80000000u;  // past the last block: zeros
         if (MT == 2) {
             const int cc = (lane & 1) ^ ((lane >> 4) & 1);
             voff_a = 16 * cc < cp.lda ? (uint32_t)((32 * wave + (lane >> 1)) * cp.lda + 16 * cc) : 0x80000000u;
@@ -509,8 +534,11 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
         const uint32_t skip_b = (uint32_t)kb * KBLOCK * (uint32_t)N;
         const uint32_t skip_a = (uint32_t)kb * KBLOCK * (uint32_t)cp.lda;
         const v4i rb = make_rsrc_words(cp.b + skip_b, b_bytes - skip_b);
-        lds_dma16(rb, voff_b[0], stage + (uint32_t)((2 * wave) * 1024));
-        lds_dma16(rb, voff_b[1], stage + (uint32_t)((2 * wave + 1) * 1024));
+#pragma unroll
+        for (int h = 0; h < NB; ++h) {
+            lds_dma16(rb, voff_b[h][0], stage + (uint32_t)(h * S::HALF_B + (2 * wave) * 1024));
+            lds_dma16(rb, voff_b[h][1], stage + (uint32_t)(h * S::HALF_B + (2 * wave + 1) * 1024));
+        }
         const int scale_wave = MT == 2 ? wave - 4 : wave;
         if (MT == 4 || wave < 4)
             lds_dma16(make_rsrc_words(cp.a + skip_a, a_bytes - skip_a), voff_a, stage + S::MAT_B + (uint32_t)(wave * 1024));
@@ -547,9 +575,9 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
         v2i r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(v2i, lds + addr + 3 * step));
         return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
     };
-    v4f acc[MT];
-    const DecodeProblem mp = one;
-    int mp_strip = 0;
+    v4f acc[NB][MT];
+    DecodeProblem mp = one;
+    int mp_strip = 0, mp_tiles = TILES;
 
 #pragma unroll
     for (int p = 0; p < DS_NS - 1; ++p)
@@ -567,42 +595,88 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
         __syncthreads();  // everyone's copies of stage t landed; the slot of stage t - 1 is no longer read
         issue_next();     // stage t + DS_NS - 1 goes into the slot of stage t - 1
         if (kb == 0) {
-            mp_strip = unit;
+            mp = problem_of(unit, &mp_strip);
+            if (TILES == 0)
+                mp_tiles = (mp.M + 15) >> 4;
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
-                acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+            for (int h = 0; h < NB; ++h)
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    acc[h][i] = (v4f){0.f, 0.f, 0.f, 0.f};
         }
         const uint32_t so = (uint32_t)(slot * S::STAGE);
-        const v8i fb = read_frag(so + addr_b, 32 * 128);
-        const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
-        // TILES 16-row tiles (fixed per launch): every read of the stage is issued before the first MFMA
-        v8i fa[TILES];
-        float sa[TILES];
+        // T 16-row tiles: every read of the stage is issued before the first MFMA, no branch among them
+        auto stage_math = [&](auto tile_count) __attribute__((always_inline)) {
+            constexpr int T = decltype(tile_count)::value;
+            v8i fb[NB], fa[T];
+            float sb[NB], sa[T];
 #pragma unroll
-        for (int i = 0; i < TILES; ++i) {
-            sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
-            fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
-        }
+            for (int h = 0; h < NB; ++h) {
+                fb[h] = read_frag(so + h * S::HALF_B + addr_b, 32 * 128);
+                sb[h] = *LDS_PTR(float, lds + so + S::SB_OFF + 4 * h);
+            }
 #pragma unroll
-        for (int i = 0; i < TILES; ++i) {
-            const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[i], (v4f){0.f, 0.f, 0.f, 0.f}, 0,
-                                                                             0, 0, 0, 0, 0);
-            const float sc = sa[i] * sb;
-            acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]), fmaf(sc, blk[2], acc[i][2]),
-                           fmaf(sc, blk[3], acc[i][3])};
-        }
+            for (int i = 0; i < T; ++i) {
+                sa[i] = *LDS_PTR(float, lds + so + S::SA_OFF + (16 * i + i16) * 4);
+                fa[i] = read_frag(so + addr_a + (uint32_t)((i ^ swz_a) * 16), 32 * S::RSA);
+            }
+#pragma unroll
+            for (int h = 0; h < NB; ++h)
+#pragma unroll
+                for (int i = 0; i < T; ++i) {
+                    const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        fb[h], fa[i], (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                    const float sc = sa[i] * sb[h];
+                    acc[h][i] = (v4f){fmaf(sc, blk[0], acc[h][i][0]), fmaf(sc, blk[1], acc[h][i][1]),
+                                      fmaf(sc, blk[2], acc[h][i][2]), fmaf(sc, blk[3], acc[h][i][3])};
+                }
+        };
+        if (TILES > 0)
+            stage_math(std::integral_constant<int, (TILES > 0 ? TILES : 1)>{});
+        else
+            switch (mp_tiles) {
+            case 1: stage_math(std::integral_constant<int, 1>{}); break;
+            case 2: stage_math(std::integral_constant<int, 2>{}); break;
+            case 3: stage_math(std::integral_constant<int, (MT == 4 ? 3 : 1)>{}); break;
+            default: stage_math(std::integral_constant<int, (MT == 4 ? 4 : 1)>{}); break;
+            }
         slot = slot == DS_NS - 1 ? 0 : slot + 1;
         if (++kb == nkb) {
-            // a lane holds C[16*i + (lane & 15)][n0 + 16*wave + 4*(lane >> 4) + 0..3]
-            const int ncol = mp_strip * DS_BN + 16 * wave + 4 * g4;
+            // a lane holds C[16*i + (lane & 15)][n0 + 128*h + 16*wave + 4*(lane >> 4) + 0..3]
+            if (STAGED) {
+                const uint32_t cbase = (uint32_t)(DS_NS * S::STAGE);
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                const int mrow = 16 * i + i16;
-                if (mrow < mp.M && ncol < N) {
-                    uint2 pk;
-                    pk.x = pack_bf16x2(acc[i][0], acc[i][1]);
-                    pk.y = pack_bf16x2(acc[i][2], acc[i][3]);
-                    *reinterpret_cast<uint2*>(mp.c + (size_t)mrow * N + ncol) = pk;
+                for (int h = 0; h < NB; ++h)
+#pragma unroll
+                    for (int i = 0; i < (TILES > 0 ? TILES : MT); ++i)
+                        if (TILES > 0 || i < mp_tiles)
+                            *LDS_PTR(v2i, lds + cbase + (16 * i + i16) * C_STAGE_ROW + (DS_BN * h + 16 * wave + 4 * g4) * 2) =
+                                (v2i){(int)pack_bf16x2(acc[h][i][0], acc[h][i][1]),
+                                      (int)pack_bf16x2(acc[h][i][2], acc[h][i][3])};
+                __syncthreads();  // (the next write to this area lies behind the next stage's barrier)
+                constexpr int CPR = BN / 8;  // 16-byte chunks per row
+                const int staged_rows = 16 * (TILES > 0 ? TILES : mp_tiles);
+                for (int idx = (int)threadIdx.x; idx < staged_rows * CPR; idx += DS_THREADS) {
+                    const int row = idx / CPR, ch = idx % CPR;
+                    const int ncol = mp_strip * BN + 8 * ch;
+                    if (row < mp.M && ncol < N)
+                        *reinterpret_cast<v4i*>(mp.c + (size_t)row * N + ncol) =
+                            *LDS_PTR(v4i, lds + cbase + row * C_STAGE_ROW + 16 * ch);
+                }
+            } else {
+#pragma unroll
+                for (int h = 0; h < NB; ++h) {
+                    const int ncol = mp_strip * BN + DS_BN * h + 16 * wave + 4 * g4;
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        const int mrow = 16 * i + i16;
+                        if (mrow < mp.M && ncol < N) {
+                            uint2 pk;
+                            pk.x = pack_bf16x2(acc[h][i][0], acc[h][i][1]);
+                            pk.y = pack_bf16x2(acc[h][i][2], acc[h][i][3]);
+                            *reinterpret_cast<uint2*>(mp.c + (size_t)mrow * N + ncol) = pk;
+                        }
+                    }
                 }
             }
             kb = 0;
@@ -611,13 +685,21 @@ __device__ __forceinline__ void decode_stream_body(const DecodeProblem& one, int
     }
 }
 
-template <int MT, int DS_NS, int TILES>
+template <int MT, int DS_NS, bool STAGED, int NB>
+__global__ void __launch_bounds__(DS_THREADS)
+decode_stream_grouped_kernel(const GroupTable tab, int N, int K, int strips, int units)
+{
+    const DecodeProblem none{};
+    decode_stream_body<MT, DS_NS, 0, STAGED, NB, true>(none, &tab, N, K, strips, units);
+}
+
+template <int MT, int DS_NS, int TILES, bool STAGED, int NB>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_stream_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
                      const float* __restrict__ b_scale, uint16_t* __restrict__ c, int M, int N, int K, int strips)
 {
     const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
-    decode_stream_body<MT, DS_NS, TILES>(one, N, K, strips);
+    decode_stream_body<MT, DS_NS, TILES, STAGED, NB, false>(one, nullptr, N, K, strips, strips);
 }
 
 // records the XCC (XCD) id each workgroup of a probe grid runs on
@@ -634,8 +716,15 @@ __global__ void xcc_probe_kernel(unsigned int* out)
 
 inline int row_tiles(int m) { return m <= 32 ? 2 : 4; }
 
-// the streaming form: ring depth and workgroups (one per CU with six stages)
+// the streaming form: ring depth and workgroups (one per CU; six stages, five beside four staged row tiles of C)
 constexpr int STREAM_NS = 6;
+constexpr int STREAM_NS4 = 5;
+constexpr int STREAM_NS_WIDE = 3;  // 256-column strips: 32 KB of B per stage
+constexpr long GROUPED_STREAM_MIN_UNITS = 256;  // grouped launches: 256-column strips of all groups for the streaming form
+template <int MT_, int NS_, int NB_>
+struct StreamShape {
+    static constexpr int MT = MT_, NS = NS_, NB = NB_;
+};
 constexpr int STREAM_WORKGROUPS = 256;
 
 // Two workgroups per CU with a three-stage ring instead of one with six: one streams while the other starts up.
@@ -732,18 +821,35 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
         return hipGetLastError();
     };
     if (ksplit == 1 && strips > STREAM_WORKGROUPS && g.m % 16 == 0) {  // more units than resident workgroups: one copy stream per workgroup
-        auto stream = [&](auto kern, int lds) -> hipError_t {
+        const bool staged = reinterpret_cast<uintptr_t>(g.c) % 16 == 0;
+        const int wide_units = (g.n + 2 * DS_BN - 1) / (2 * DS_BN);
+        const bool wide = wide_units >= STREAM_WORKGROUPS;  // 256-column strips while every CU gets one
+        const int units = wide ? wide_units : strips;
+        auto stream = [&](auto shape, auto tiles_c, auto staged_c) -> hipError_t {
+            constexpr int MT = decltype(shape)::MT, NS = decltype(shape)::NS, NB = decltype(shape)::NB;
+            constexpr int T = decltype(tiles_c)::value;
+            constexpr bool ST = decltype(staged_c)::value;
+            constexpr int lds = DecodeShape<MT, NS, false, NB>::LDS + (ST ? 16 * T * (2 * DS_BN * NB + 16) : 0);
+            static_assert(lds <= 160 * 1024, "ring and staged C exceed the LDS");
+            auto kern = decode_stream_kernel<MT, NS, T, ST, NB>;
             FP8GEMM_ALLOW_LDS(kern, lds);
             hipLaunchKernelGGL(kern, dim3(STREAM_WORKGROUPS), dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
-                               g.m, g.n, g.k, strips);
+                               g.m, g.n, g.k, units);
             return hipGetLastError();
         };
-        switch (g.m / 16) {
-        case 1: return stream(decode_stream_kernel<2, STREAM_NS, 1>, DecodeShape<2, STREAM_NS>::LDS);
-        case 2: return stream(decode_stream_kernel<2, STREAM_NS, 2>, DecodeShape<2, STREAM_NS>::LDS);
-        case 3: return stream(decode_stream_kernel<4, STREAM_NS, 3>, DecodeShape<4, STREAM_NS>::LDS);
-        default: return stream(decode_stream_kernel<4, STREAM_NS, 4>, DecodeShape<4, STREAM_NS>::LDS);
-        }
+        auto by_staging = [&](auto shape, auto tiles_c) -> hipError_t {
+            return staged ? stream(shape, tiles_c, std::true_type{}) : stream(shape, tiles_c, std::false_type{});
+        };
+        auto by_tiles = [&](auto shape2, auto shape4) -> hipError_t {
+            switch (g.m / 16) {
+            case 1: return by_staging(shape2, std::integral_constant<int, 1>{});
+            case 2: return by_staging(shape2, std::integral_constant<int, 2>{});
+            case 3: return by_staging(shape4, std::integral_constant<int, 3>{});
+            default: return by_staging(shape4, std::integral_constant<int, 4>{});
+            }
+        };
+        return wide ? by_tiles(StreamShape<2, STREAM_NS_WIDE, 2>{}, StreamShape<4, STREAM_NS_WIDE, 2>{})
+                    : by_tiles(StreamShape<2, STREAM_NS, 1>{}, StreamShape<4, STREAM_NS4, 1>{});
     }
     const int tiles = (g.m + 15) / 16;
     if (g.m % 16 != 0) {
@@ -814,6 +920,16 @@ int decode_grouped_ksplit(const GroupTable& tab, int n, int k, bool fused_ok)
     return best;
 }
 
+// Whether a grouped launch of this many groups is one for the streaming form with 256-column strips: 256
+// workgroups take the units in turn, which pays while the last turn is not too empty (288 units are two turns for
+// 56 % of the work of two: 145 us against 121 us for 16 x (4608 x 7168); 448 units: 44 against 49 us).
+bool decode_grouped_streams(int groups, int n)
+{
+    const long wide_units = (long)((n + 2 * DS_BN - 1) / (2 * DS_BN)) * groups;
+    const long turns = (wide_units + STREAM_WORKGROUPS - 1) / STREAM_WORKGROUPS;
+    return wide_units >= GROUPED_STREAM_MIN_UNITS && 5 * wide_units >= 4 * turns * STREAM_WORKGROUPS;
+}
+
 hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit, float* mailbox, hipStream_t s)
 {
     const int strips = (n + DS_BN - 1) / DS_BN;
@@ -831,6 +947,30 @@ hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit
     for (int g = 0; g < tab.groups; ++g) {
         mmax = tab.lda[g] > mmax ? tab.lda[g] : mmax;
         ragged |= tab.lda[g] % 16 != 0;
+    }
+    // many strips, rows on the 16-byte grid, no K split: the streaming form with 256-column strips
+    const int wide_strips = (n + 2 * DS_BN - 1) / (2 * DS_BN);
+    const long wide_units = (long)wide_strips * tab.groups;
+    if (ksplit == 1 && !ragged && decode_grouped_streams(tab.groups, n)) {
+        bool staged = true;
+        for (int g = 0; g < tab.groups; ++g)
+            staged = staged && reinterpret_cast<uintptr_t>(tab.c[g]) % 16 == 0;
+        auto stream = [&](auto shape, auto staged_c) -> hipError_t {
+            constexpr int MT = decltype(shape)::MT, NS = decltype(shape)::NS, NB = decltype(shape)::NB;
+            constexpr bool ST = decltype(staged_c)::value;
+            constexpr int lds = DecodeShape<MT, NS, false, NB>::LDS + (ST ? 16 * MT * (2 * DS_BN * NB + 16) : 0);
+            static_assert(lds <= 160 * 1024, "ring and staged C exceed the LDS");
+            auto kern = decode_stream_grouped_kernel<MT, NS, ST, NB>;
+            FP8GEMM_ALLOW_LDS(kern, lds);
+            hipLaunchKernelGGL(kern, dim3(STREAM_WORKGROUPS), dim3(DS_THREADS), lds, s, tab, n, k, wide_strips,
+                               (int)wide_units);
+            return hipGetLastError();
+        };
+        if (row_tiles(mmax) == 2)
+            return staged ? stream(StreamShape<2, STREAM_NS_WIDE, 2>{}, std::true_type{})
+                          : stream(StreamShape<2, STREAM_NS_WIDE, 2>{}, std::false_type{});
+        return staged ? stream(StreamShape<4, STREAM_NS_WIDE, 2>{}, std::true_type{})
+                      : stream(StreamShape<4, STREAM_NS_WIDE, 2>{}, std::false_type{});
     }
     const dim3 grid((unsigned)(8 * ((units + 7) / 8) * ksplit));
     auto go = [&](auto kern, int lds) -> hipError_t {

@@ -105,6 +105,7 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
 bool decode_grouped_supports(const GroupTable& tab, int n, int k);
 int decode_grouped_ksplit(const GroupTable& tab, int n, int k, bool fused_ok);
 size_t decode_grouped_mailbox_bytes(const GroupTable& tab, int n, int ksplit);
+bool decode_grouped_streams(int groups, int n);  // the launch takes the streaming form (rows on the 16-byte grid, no K split)
 hipError_t launch_decode_grouped(const GroupTable& tab, int n, int k, int ksplit, float* mailbox, hipStream_t s);
 // 1 = workgroups whose linear ids agree modulo 8 share an XCD on the current device (looked at once
 // per device with a probe grid, which the first call waits for: not under stream capture),

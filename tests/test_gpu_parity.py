@@ -243,7 +243,10 @@ DECODE_STRIP_CASES = [(32, 7168, 2048, 4), (16, 7168, 2048, 4), (32, 7168, 2048,
                       (32, 7168, 7168, 8),
                       # more strips than the device holds workgroups, no K split: the streaming form (a workgroup
                       # walks through several strips, one copy stream); ragged last strip; a single K block
-                      (16, 33040, 384, 1), (32, 40960, 256, 1), (48, 33024, 128, 1)]
+                      (16, 33040, 384, 1), (32, 40960, 256, 1), (48, 33024, 128, 1),
+                      # wide enough for 256-column strips on every CU: full strips, a last strip that ends in its
+                      # first half, one that ends in its second, one to four row tiles
+                      (32, 65536, 256, 1), (16, 65616, 384, 1), (64, 65744, 128, 1), (48, 66000, 256, 1)]
 
 
 @pytest.mark.parametrize("m,n,k,ksplit", DECODE_STRIP_CASES)
@@ -870,13 +873,15 @@ def test_grouped_decode_groups_equal_the_problems_one_by_one(pkg, ms, n, k):
 
 def test_grouped_decode_groups_off_the_16_byte_grid_and_mixed_with_tall_groups(pkg):
     """ragged token counts of 1 to 64 rows run in one decode launch (on padded copies only when n is off the
-    grid); a
+    grid, or the launch is large enough for the streaming form); a
     call that also holds taller groups launches the tile kernel for those; rows beyond m stay untouched"""
     import torch
     st = torch.cuda.current_stream().cuda_stream
     for ms, n, k in [([1, 7, 64, 33, 16, 50, 2], 1536, 1024), ([5, 300, 64, 1000, 17], 640, 512), ([3, 9], 200, 256),
                      # more than one round of workgroups; more K blocks than ring slots
-                     ([3, 16, 9, 1] * 6, 2048, 384), ([17, 31, 5, 20] * 5, 2048, 384), ([20, 7], 256, 3328)]:
+                     ([3, 16, 9, 1] * 6, 2048, 384), ([17, 31, 5, 20] * 5, 2048, 384), ([20, 7], 256, 3328),
+                     # enough 256-column strips for the streaming form, which wants rows on the grid: padded copies of A
+                     ([1 + (7 * g) % 40 for g in range(64)], 2048, 256)]:
         host, dev, outs = [], [], []
         for g, m in enumerate(ms):
             a, b, sa, sb = oracle.make_inputs(m, n, k, 9300 + 11 * g + n)
@@ -888,7 +893,9 @@ def test_grouped_decode_groups_off_the_16_byte_grid_and_mixed_with_tall_groups(p
                          outs, ms, n, k, st)
         torch.cuda.synchronize()
         name = pkg.last_kernel()
-        assert "decode128_k" in name and name.startswith("padded_decode128_k") == (n % 16 != 0), name
+        wide_units = sum(1 for m in ms if m <= 64) * -(-n // 256)
+        streams = wide_units >= 256 and 5 * wide_units >= 4 * -(-wide_units // 256) * 256
+        assert "decode128_k" in name and name.startswith("padded_decode128_k") == (n % 16 != 0 or streams), name
         if max(ms) > 64:
             assert "+" in name and "tile" in name, name
         for g, m in enumerate(ms):
