@@ -133,7 +133,9 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * layer in a decode step) do not go through 128-row tiles: they run as ONE launch of the decode kernel
  * ("decode128_kN_groupedG": 128-column strips of every group in one work list, every group's B read
  * once, the K range split and added inside the kernel as for a single problem; row counts off the 16-row
- * grid as they are, without copies); a call that mixes both kinds launches each kernel once.  More groups than FP8GEMM_MAX_GROUPS fall back to one call
+ * grid as they are, without copies, except in launches large enough for the streaming form -- 256 or more
+ * strips of 256 columns over all groups --, which runs on padded copies of A and a_scale); a call that mixes
+ * both kinds launches each kernel once.  More groups than FP8GEMM_MAX_GROUPS fall back to one call
  * of fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to
  * what fp8_block_gemm_stream gives for that problem with the same tile shape (decode kernel: with the
  * same K split).  No counterpart in the
