@@ -98,6 +98,7 @@ struct Plan {
     bool padded = false;      // the plan is for the problem with m and n rounded up to 16 (run_padded)
     bool wide = false;        // decode family: 128-column strips, K splits added inside the kernel (k_decode.hip)
     bool fused = false;       // tile family, ksplit > 1: the last workgroup of a tile adds the partial tiles (no reduction launch)
+    int halves = 1;           // wide decode strips: 128-column halves per strip (2 = 256-column strips)
 };
 
 // Shapes or addresses the MFMA kernels cannot take (m or n not a multiple of 16, a base not
@@ -282,21 +283,29 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
         double narrow_us = 1e300, wide_us = 1e300;
         Plan narrow = decode, wide = decode;
         wide.wide = true;
-        if (narrow_ok && !(by_name && cfg.force_variant == 1)) {
+        if (narrow_ok && !(by_name && cfg.force_variant >= 1)) {
             narrow.ksplit = forced_ks ? forced_ks : skinny_ksplit(g);
             narrow_us = skinny_cost(g, narrow.ksplit);
         }
         if (wide_ok && (by_name ? cfg.force_variant != 0 : cfg.force_variant < 0)) {
             // without the in-kernel reduction (no zeroed mailbox, or workgroup placement not confirmed) only
-            // the unsplit form exists
+            // the unsplit form exists.  By name, tile_variant 2 pins the 256-column strips.
+            // Left to the cost model, 256-column strips have to be 7 % ahead: they halve the workgroups of a
+            // split and win where that saves a round (144 strips x 3 splits are 54 workgroups on an XCD's 32 CUs,
+            // 72 x 3 are 27: 18432 x 7168 from HBM 28.6 against 34.6 us), and lose 15 - 40 % on cfg5-sized problems.
             const int hi = cfg.fused_ok ? (nkb < MAX_KSPLIT ? nkb : MAX_KSPLIT) : 1;
-            for (int ks = 1; ks <= hi; ++ks) {
-                if (!valid_split(ks) || (forced_ks && ks != forced_ks) || !decode_strip_can_split(g, ks))
+            for (int halves = 1; halves <= 2; ++halves) {
+                if (by_name ? halves != (cfg.force_variant == 2 ? 2 : 1) : cfg.force_variant >= 0 && halves == 2)
                     continue;
-                const double cst = decode_strip_cost(g, ks);
-                if (cst < wide_us) {
-                    wide_us = cst;
-                    wide.ksplit = ks;
+                for (int ks = 1; ks <= hi; ++ks) {
+                    if (!valid_split(ks) || (forced_ks && ks != forced_ks) || !decode_strip_can_split(g, ks, halves))
+                        continue;
+                    const double cst = decode_strip_cost(g, ks, halves) * (halves == 2 && !by_name ? 1.07 : 1.0);
+                    if (cst < wide_us) {
+                        wide_us = cst;
+                        wide.ksplit = ks;
+                        wide.halves = halves;
+                    }
                 }
             }
         }
@@ -509,7 +518,7 @@ void plan_name(const Plan& p, char* out, size_t cap)
     if (p.family == FP8GEMM_KERNEL_SCALAR)
         snprintf(out, cap, "scalar");
     else if (p.family == FP8GEMM_KERNEL_SKINNY)
-        snprintf(out, cap, p.wide ? "%sdecode128_k%d" : "%sskinny_k%d", pre, p.ksplit);
+        snprintf(out, cap, p.wide ? (p.halves == 2 ? "%sdecode256_k%d" : "%sdecode128_k%d") : "%sskinny_k%d", pre, p.ksplit);
     else
         snprintf(out, cap, "%s%s_k%d%s", pre, tile_variant_name(p.variant), p.ksplit,
                  p.persistent ? "_persistent" : (p.fused ? "f" : ""));
@@ -524,7 +533,7 @@ hipError_t launch_plan(const GemmArgs& g, const Plan& p, float* partial, const W
         return launch_scalar(g, stream);
     case FP8GEMM_KERNEL_SKINNY:
         if (p.wide)
-            return launch_decode_strips(g, p.ksplit, ws_mailbox(w), stream);
+            return launch_decode_strips(g, p.ksplit, p.halves, ws_mailbox(w), stream);
         return launch_skinny(g, p.ksplit, partial, stream);
     default: {
         if (p.persistent)
@@ -623,7 +632,7 @@ int run(const void* a, const void* b, const float* as, const float* bs, void* c,
         probe.fused_ok = false;
         const Plan with = make_plan(g, cfg), without = make_plan(g, probe);
         const bool differs = with.family != without.family || with.ksplit != without.ksplit ||
-                             with.wide != without.wide || with.fused != without.fused;
+                             with.wide != without.wide || with.fused != without.fused || with.halves != without.halves;
         if (differs && !placement_ok(stream))
             cfg.fused_ok = false;
     }

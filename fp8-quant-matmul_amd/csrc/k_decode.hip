@@ -112,11 +112,12 @@ struct DecodeProblem {
 // with u = grp * 8 + xcd.
 // TILES = the number of 16-row tiles when the launch knows it (a single problem: the count is then a constant
 // in the epilogue as well), 0 = read from the problem (grouped launches).
-template <int MT, bool GROUPED, int DS_NS, bool RAGGED, int TILES>
+template <int MT, bool GROUPED, int DS_NS, bool RAGGED, int TILES, int NB>
 __device__ __forceinline__ void decode_body(const DecodeProblem& one, const GroupTable* tab, float* mailbox, int N, int K,
                                             int strips, int units, int ksplit, int kb_per_split)
 {
-    using S = DecodeShape<MT, DS_NS, RAGGED>;
+    using S = DecodeShape<MT, DS_NS, RAGGED, NB>;
+    constexpr int BN = DS_BN * NB;  // columns of a strip
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     auto lds = LDS_PTR(uint8_t, smem);
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -143,7 +144,7 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     const float* __restrict__ b_scale = pr.b_scale;
     uint16_t* __restrict__ c = pr.c;
     const int M = pr.M, lda = pr.lda;
-    const int n0 = strip * DS_BN;
+    const int n0 = strip * BN;
 
     const int nkb = K / KBLOCK;
     const int kb0 = split * kb_per_split;
@@ -156,15 +157,17 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
     // 0..3, rows 32*wave + (lane >> 1), position lane & 1, swizzle (r >> 3) & 1 = (lane >> 4) & 1; 64-byte
     // rows: every wave, rows 16*wave + (lane >> 2), position lane & 3, swizzle (r >> 2) & 3 = (lane >> 4) & 3.
     const uint32_t a_bytes = (uint32_t)lda * (uint32_t)K, b_bytes = (uint32_t)N * (uint32_t)K;
-    uint32_t voff_b[2];
+    uint32_t voff_b[NB][2];  // per 128-column half of the strip
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int cc = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
-        const bool ok = n0 + 16 * cc < N;
-        voff_b[q] = ok ? (uint32_t)((16 * wave + 8 * q + (lane >> 3)) * N + n0 + 16 * cc) : 0x80000000u;
-    }
+    for (int h = 0; h < NB; ++h)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int cc = (lane & 7) ^ ((4 * q + (lane >> 4)) & 7);
+            const bool ok = n0 + DS_BN * h + 16 * cc < N;
+            voff_b[h][q] = ok ? (uint32_t)((16 * wave + 8 * q + (lane >> 3)) * N + n0 + DS_BN * h + 16 * cc) : 0x80000000u;
+        }
     const uint32_t voff_sa = lane < lda ? (uint32_t)(lane * 4) : 0x80000000u;
-    const uint32_t voff_sb = lane == 0 ? (uint32_t)(strip * 4) : 0x80000000u;
+    const uint32_t voff_sb = lane < NB ? (uint32_t)((strip * NB + lane) * 4) : 0x80000000u;  // past the last block: zeros
     uint32_t voff_a;
     if (RAGGED) {
         // the K block's slab of A, 128 * M contiguous bytes, in 16-byte pieces: piece 64 * wave + lane
@@ -184,8 +187,11 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         const uint32_t skip_b = (uint32_t)kb * KBLOCK * (uint32_t)N;
         const uint32_t skip_a = (uint32_t)kb * KBLOCK * (uint32_t)lda;
         const v4i rb = make_rsrc_words(b + skip_b, b_bytes - skip_b);
-        lds_dma16(rb, voff_b[0], stage + (uint32_t)((2 * wave) * 1024));
-        lds_dma16(rb, voff_b[1], stage + (uint32_t)((2 * wave + 1) * 1024));
+#pragma unroll
+        for (int h = 0; h < NB; ++h) {
+            lds_dma16(rb, voff_b[h][0], stage + (uint32_t)(h * S::HALF_B + (2 * wave) * 1024));
+            lds_dma16(rb, voff_b[h][1], stage + (uint32_t)(h * S::HALF_B + (2 * wave + 1) * 1024));
+        }
         const int scale_wave = MT == 2 ? wave - 4 : wave;  // 0: a_scale, 1..: b_scale, below 0: A (two row tiles)
         if (RAGGED) {
             // the slab of the K block after this one, into the next slot: it has landed with this stage, one
@@ -263,10 +269,12 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         return (v8i){r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
     };
 
-    v4f acc[MT];
+    v4f acc[NB][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-        acc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < NB; ++h)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            acc[h][i] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int nstages = kb1 - kb0;
     if (RAGGED && (MT == 4 || wave < 4)) {  // the first K block's slab, ahead of every stage
@@ -302,14 +310,19 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         // RAGGED: the next stage's slab, also behind the last stage (nothing reads what that spreads)
         if (RAGGED)
             slab_read(next_slot);
-        const v8i fb = read_frag(so + addr_b, 32 * 128);
-        const float sb = *LDS_PTR(float, lds + so + S::SB_OFF);
-        auto multiply = [&](int i, const v8i& fa, float sa) __attribute__((always_inline)) {
-            const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0,
-                                                                             0, 0, 0);
-            const float sc = sa * sb;
-            acc[i] = (v4f){fmaf(sc, blk[0], acc[i][0]), fmaf(sc, blk[1], acc[i][1]), fmaf(sc, blk[2], acc[i][2]),
-                           fmaf(sc, blk[3], acc[i][3])};
+        v8i fb[NB];
+        float sb[NB];
+#pragma unroll
+        for (int h = 0; h < NB; ++h) {
+            fb[h] = read_frag(so + h * S::HALF_B + addr_b, 32 * 128);
+            sb[h] = *LDS_PTR(float, lds + so + S::SB_OFF + 4 * h);
+        }
+        auto multiply = [&](int h, int i, const v8i& fa, float sa) __attribute__((always_inline)) {
+            const v4f blk = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[h], fa, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0,
+                                                                             0, 0, 0, 0);
+            const float sc = sa * sb[h];
+            acc[h][i] = (v4f){fmaf(sc, blk[0], acc[h][i][0]), fmaf(sc, blk[1], acc[h][i][1]),
+                              fmaf(sc, blk[2], acc[h][i][2]), fmaf(sc, blk[3], acc[h][i][3])};
         };
         // the spread words are written behind the stage's reads: the LDS works in order, a write among the
         // reads would hold the later ones back
@@ -323,8 +336,10 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         if (RAGGED)
             slab_write(next_slot);
 #pragma unroll
-        for (int i = 0; i < T; ++i)
-            multiply(i, fa[i], sa[i]);
+        for (int h = 0; h < NB; ++h)
+#pragma unroll
+            for (int i = 0; i < T; ++i)
+                multiply(h, i, fa[i], sa[i]);
         slot = next_slot;
     }
     };
@@ -344,17 +359,20 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         break;
     }
 
-    // ---- a lane holds C[16*i + (lane & 15)][n0 + 16*wave + 4*(lane >> 4) + 0..3]
-    const int ncol = n0 + 16 * wave + 4 * g4;
-    auto store_c = [&](const v4f (&v)[MT]) __attribute__((always_inline)) {
+    // ---- a lane holds C[16*i + (lane & 15)][n0 + 128*h + 16*wave + 4*(lane >> 4) + 0..3]
+    auto store_c = [&](const v4f (&v)[NB][MT]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int mrow = 16 * i + i16;
-            if (mrow < M && ncol < N) {
-                uint2 pk;
-                pk.x = pack_bf16x2(v[i][0], v[i][1]);
-                pk.y = pack_bf16x2(v[i][2], v[i][3]);
-                *reinterpret_cast<uint2*>(c + (size_t)mrow * N + ncol) = pk;
+        for (int h = 0; h < NB; ++h) {
+            const int ncol = n0 + DS_BN * h + 16 * wave + 4 * g4;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const int mrow = 16 * i + i16;
+                if (mrow < M && ncol < N) {
+                    uint2 pk;
+                    pk.x = pack_bf16x2(v[h][i][0], v[h][i][1]);
+                    pk.y = pack_bf16x2(v[h][i][2], v[h][i][3]);
+                    *reinterpret_cast<uint2*>(c + (size_t)mrow * N + ncol) = pk;
+                }
             }
         }
     };
@@ -363,35 +381,41 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
         return;
     }
 
-    // ---- mailbox: [unit][split 0 .. ksplit-2][wave][i][lane] x 16 bytes, all zero between launches
-    constexpr int PER_SPLIT = 8 * MT;  // patches of one split of one unit
+    // ---- mailbox: [unit][split 0 .. ksplit-2][wave][half h][i][lane] x 16 bytes, all zero between launches
+    constexpr int PER_WAVE = NB * MT;        // patches of one wave
+    constexpr int PER_SPLIT = 8 * PER_WAVE;  // patches of one split of one unit
     const int senders = ksplit - 1;
-    const size_t patch = ((size_t)unit * senders * 8 + wave) * MT;  // split 0
+    const size_t patch = ((size_t)unit * senders * 8 + wave) * PER_WAVE;  // split 0
     if (split < senders) {
         v4i* mine = reinterpret_cast<v4i*>(mailbox) + (patch + (size_t)split * PER_SPLIT) * 64 + lane;
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-            if (i < mtiles) {
-                v4i bits = __builtin_bit_cast(v4i, acc[i]);
+        for (int h = 0; h < NB; ++h)
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    bits[e] = bits[e] == 0 ? (int)0x80000000 : bits[e];  // +0.0 -> -0.0: no word is zero
-                mine[64 * i] = bits;
-            }
+            for (int i = 0; i < MT; ++i)
+                if (i < mtiles) {
+                    v4i bits = __builtin_bit_cast(v4i, acc[h][i]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        bits[e] = bits[e] == 0 ? (int)0x80000000 : bits[e];  // +0.0 -> -0.0: no word is zero
+                    mine[64 * (h * MT + i)] = bits;
+                }
         return;
     }
     // last split: wait for the other splits' patches of these 16 columns, four splits at a time
     const uint32_t span = (uint32_t)senders * PER_SPLIT * 64u * 16u;  // bytes from this wave's split-0 patch to past its last
     const __amdgpu_buffer_rsrc_t rp = make_rsrc(reinterpret_cast<const v4i*>(mailbox) + patch * 64, span);
-    v4f sum[MT];
+    v4f sum[NB][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-        sum[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < NB; ++h)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            sum[h][i] = (v4f){0.f, 0.f, 0.f, 0.f};
     bool gave_up = false;
     const unsigned long long t_first = __builtin_amdgcn_s_memrealtime();
     for (int z0 = 0; z0 < senders; z0 += 4) {
 #pragma unroll
-        for (int h = 0; h < MT / 2; ++h) {  // two row tiles at a time
+        for (int hp = 0; hp < NB * (MT / 2); ++hp) {  // two row tiles of a half at a time
+            const int hb = hp / (MT / 2), h = hp % (MT / 2);
             if (2 * h < mtiles) {
                 v4i v[4][2];
                 for (;;) {
@@ -402,7 +426,7 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
 #pragma unroll
                         for (int i = 0; i < 2; ++i)
                             v[z][i] = __builtin_amdgcn_raw_buffer_load_b128(
-                                rp, (uint32_t)(((z0 + z) * PER_SPLIT + 2 * h + i) * 64 + lane) * 16u, 0, AUX_L1_MISS);
+                                rp, (uint32_t)(((z0 + z) * PER_SPLIT + hb * MT + 2 * h + i) * 64 + lane) * 16u, 0, AUX_L1_MISS);
                     bool missing = false;
 #pragma unroll
                     for (int z = 0; z < 4; ++z)
@@ -424,31 +448,34 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
                         for (int i = 0; i < 2; ++i) {
                             if (2 * h + i < mtiles)
                                 __builtin_amdgcn_raw_buffer_store_b128(
-                                    (v4i){0, 0, 0, 0}, rp, (uint32_t)(((z0 + z) * PER_SPLIT + 2 * h + i) * 64 + lane) * 16u, 0, 0);
+                                    (v4i){0, 0, 0, 0}, rp,
+                                    (uint32_t)(((z0 + z) * PER_SPLIT + hb * MT + 2 * h + i) * 64 + lane) * 16u, 0, 0);
                             const v4f f = __builtin_bit_cast(v4f, v[z][i]);
-                            sum[2 * h + i] = z0 + z == 0 ? f : sum[2 * h + i] + f;
+                            sum[hb][2 * h + i] = z0 + z == 0 ? f : sum[hb][2 * h + i] + f;
                         }
                     }
             }
         }
     }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        sum[i] = sum[i] + acc[i];
-        if (gave_up)
-            sum[i] = (v4f){__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
-    }
+    for (int h = 0; h < NB; ++h)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            sum[h][i] = sum[h][i] + acc[h][i];
+            if (gave_up)
+                sum[h][i] = (v4f){__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+        }
     store_c(sum);
 }
 
-template <int MT, int DS_NS, bool RAGGED, int TILES>
+template <int MT, int DS_NS, bool RAGGED, int TILES, int NB>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int N, int K,
                     int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
-    decode_body<MT, false, DS_NS, RAGGED, TILES>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
+    decode_body<MT, false, DS_NS, RAGGED, TILES, NB>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
 }
 
 template <int MT, int DS_NS, bool RAGGED>
@@ -456,7 +483,7 @@ __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_grouped_kernel(const GroupTable tab, float* mailbox, int N, int K, int strips, int ksplit, int kb_per_split)
 {
     const DecodeProblem none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
-    decode_body<MT, true, DS_NS, RAGGED, 0>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
+    decode_body<MT, true, DS_NS, RAGGED, 0, 1>(none, &tab, mailbox, N, K, strips, strips * tab.groups, ksplit, kb_per_split);
 }
 
 // The streaming form, for a single problem without a K split whose strips outnumber the workgroups the
@@ -744,22 +771,25 @@ bool decode_strip_supports(const GemmArgs& g)
 }
 
 // the mailbox of a K split: one patch per strip, sending split, wave and row tile
-bool decode_strip_can_split(const GemmArgs& g, int ksplit) { return decode_strip_mailbox_bytes(g, ksplit) <= SPLIT_MAILBOX_BYTES; }
+bool decode_strip_can_split(const GemmArgs& g, int ksplit, int halves)
+{
+    return decode_strip_mailbox_bytes(g, ksplit, halves) <= SPLIT_MAILBOX_BYTES;
+}
 
-size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit)
+size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit, int halves)
 {
     if (ksplit <= 1)
         return 0;
-    const size_t strips = (size_t)(g.n + DS_BN - 1) / DS_BN;
-    return strips * (size_t)(ksplit - 1) * 8 * row_tiles(g.m) * 64 * 16;
+    const size_t strips = (size_t)(g.n + DS_BN * halves - 1) / (DS_BN * halves);
+    return strips * (size_t)(ksplit - 1) * 8 * halves * row_tiles(g.m) * 64 * 16;
 }
 // Microseconds with B streamed from HBM, fitted to M = 16 and 32, N = 1536 ... 16384, K = 1536 ... 7168 and
 // 1 to 16 K splits: a launch, then rounds of 256 workgroups, each workgroup living for a start-up, its
 // K blocks (0.5 us per block when few workgroups pull on HBM, 0.76 us when 256 do) and, when K is split,
 // the in-kernel reduction, whose last split reads one partial patch per other split.
-double decode_strip_cost(const GemmArgs& g, int ksplit)
+double decode_strip_cost(const GemmArgs& g, int ksplit, int halves)
 {
-    const int strips = (g.n + DS_BN - 1) / DS_BN;
+    const int strips = (g.n + DS_BN * halves - 1) / (DS_BN * halves);
     const int nkb = g.k / KBLOCK;
     const int kbs = (nkb + ksplit - 1) / ksplit;
     const long wgs = (long)strips * ksplit;
@@ -768,7 +798,8 @@ double decode_strip_cost(const GemmArgs& g, int ksplit)
     // 19.8 us against 14.0 us with 6 splits for 4608 x 7168)
     const long rounds = ((long)((strips + 7) / 8) * ksplit + 31) / 32;
     const double active = wgs < 256 ? (double)wgs : 256.0;
-    const double per_block = 0.50 + 0.001 * active;
+    // (a stage of a 256-column strip is twice the bytes for 1.92 times the time)
+    const double per_block = (0.50 + 0.001 * active) * (halves == 2 ? 1.92 : 1.0);
     const double life = 1.0 + kbs * per_block + (ksplit > 1 ? 0.39 * ksplit : 0.0);
     return 2.5 + (double)rounds * life;
 }
@@ -803,12 +834,14 @@ int xcd_placement_confirmed(bool may_probe)
     return ok;
 }
 
-hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, hipStream_t s)
+hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, int halves, float* mailbox, hipStream_t s)
 {
-    const int strips = (g.n + DS_BN - 1) / DS_BN;
+    if (halves != 1 && halves != 2)
+        return hipErrorInvalidValue;
+    const int strips = (g.n + DS_BN * halves - 1) / (DS_BN * halves);
     const int nkb = g.k / KBLOCK;
     if (!decode_strip_supports(g) || ksplit < 1 || ksplit > nkb || ksplit > DECODE_MAX_KSPLIT ||
-        (ksplit > 1 && (!mailbox || !decode_strip_can_split(g, ksplit))))
+        (ksplit > 1 && (!mailbox || !decode_strip_can_split(g, ksplit, halves))))
         return hipErrorInvalidValue;
     const int kb_per_split = (nkb + ksplit - 1) / ksplit;
     if ((ksplit - 1) * kb_per_split >= nkb)  // every split owns at least one K block
@@ -820,6 +853,23 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
                            g.k, strips, ksplit, kb_per_split);
         return hipGetLastError();
     };
+    if (halves == 2) {  // 256-column strips: three stages of 32 KB of B
+        const int tiles = (g.m + 15) / 16;
+        auto wide = [&](auto mt_c, auto ragged_c, auto tiles_c) -> hipError_t {
+            constexpr int MT = decltype(mt_c)::value, T = decltype(tiles_c)::value;
+            constexpr bool RG = decltype(ragged_c)::value;
+            return go(decode_strip_kernel<MT, STREAM_NS_WIDE, RG, T, 2>, DecodeShape<MT, STREAM_NS_WIDE, RG, 2>::LDS);
+        };
+        auto by_tiles = [&](auto ragged_c) -> hipError_t {
+            switch (tiles) {
+            case 1: return wide(std::integral_constant<int, 2>{}, ragged_c, std::integral_constant<int, 1>{});
+            case 2: return wide(std::integral_constant<int, 2>{}, ragged_c, std::integral_constant<int, 2>{});
+            case 3: return wide(std::integral_constant<int, 4>{}, ragged_c, std::integral_constant<int, 3>{});
+            default: return wide(std::integral_constant<int, 4>{}, ragged_c, std::integral_constant<int, 4>{});
+            }
+        };
+        return g.m % 16 != 0 ? by_tiles(std::true_type{}) : by_tiles(std::false_type{});
+    }
     if (ksplit == 1 && strips > STREAM_WORKGROUPS && g.m % 16 == 0) {  // more units than resident workgroups: one copy stream per workgroup
         const bool staged = reinterpret_cast<uintptr_t>(g.c) % 16 == 0;
         const int wide_units = (g.n + 2 * DS_BN - 1) / (2 * DS_BN);
@@ -855,20 +905,20 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, h
     if (g.m % 16 != 0) {
         constexpr int L2 = DecodeShape<2, 6, true>::LDS, L4 = DecodeShape<4, RAGGED4_NS, true>::LDS;
         switch (tiles) {
-        case 1: return go(decode_strip_kernel<2, 6, true, 1>, L2);
-        case 2: return go(decode_strip_kernel<2, 6, true, 2>, L2);
-        case 3: return go(decode_strip_kernel<4, RAGGED4_NS, true, 3>, L4);
-        default: return go(decode_strip_kernel<4, RAGGED4_NS, true, 4>, L4);
+        case 1: return go(decode_strip_kernel<2, 6, true, 1, 1>, L2);
+        case 2: return go(decode_strip_kernel<2, 6, true, 2, 1>, L2);
+        case 3: return go(decode_strip_kernel<4, RAGGED4_NS, true, 3, 1>, L4);
+        default: return go(decode_strip_kernel<4, RAGGED4_NS, true, 4, 1>, L4);
         }
     }
     const bool deep = !shallow_ring_pays((long)strips * ksplit, kb_per_split);
     constexpr int D2 = DecodeShape<2, 6>::LDS, S2 = DecodeShape<2, 3>::LDS, D4 = DecodeShape<4, 6>::LDS,
                   S4 = DecodeShape<4, 3>::LDS;
     switch (tiles) {
-    case 1: return deep ? go(decode_strip_kernel<2, 6, false, 1>, D2) : go(decode_strip_kernel<2, 3, false, 1>, S2);
-    case 2: return deep ? go(decode_strip_kernel<2, 6, false, 2>, D2) : go(decode_strip_kernel<2, 3, false, 2>, S2);
-    case 3: return deep ? go(decode_strip_kernel<4, 6, false, 3>, D4) : go(decode_strip_kernel<4, 3, false, 3>, S4);
-    default: return deep ? go(decode_strip_kernel<4, 6, false, 4>, D4) : go(decode_strip_kernel<4, 3, false, 4>, S4);
+    case 1: return deep ? go(decode_strip_kernel<2, 6, false, 1, 1>, D2) : go(decode_strip_kernel<2, 3, false, 1, 1>, S2);
+    case 2: return deep ? go(decode_strip_kernel<2, 6, false, 2, 1>, D2) : go(decode_strip_kernel<2, 3, false, 2, 1>, S2);
+    case 3: return deep ? go(decode_strip_kernel<4, 6, false, 3, 1>, D4) : go(decode_strip_kernel<4, 3, false, 3, 1>, S4);
+    default: return deep ? go(decode_strip_kernel<4, 6, false, 4, 1>, D4) : go(decode_strip_kernel<4, 3, false, 4, 1>, S4);
     }
 }
 

@@ -96,10 +96,11 @@ hipError_t launch_skinny(const GemmArgs& g, int ksplit, float* partial, hipStrea
 // decode_strip_can_split.
 constexpr int DECODE_MAX_KSPLIT = 16;
 bool decode_strip_supports(const GemmArgs& g);
-size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit);
-bool decode_strip_can_split(const GemmArgs& g, int ksplit);
-double decode_strip_cost(const GemmArgs& g, int ksplit);
-hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, float* mailbox, hipStream_t s);
+// halves = 128-column halves of a strip: 1, or 2 (256-column strips: 256 contiguous bytes of every k-row of B)
+size_t decode_strip_mailbox_bytes(const GemmArgs& g, int ksplit, int halves = 1);
+bool decode_strip_can_split(const GemmArgs& g, int ksplit, int halves = 1);
+double decode_strip_cost(const GemmArgs& g, int ksplit, int halves = 1);
+hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, int halves, float* mailbox, hipStream_t s);
 // The same kernel on several problems with common n and k and their own m <= 64 (multiples of 16), whose
 // strips form one list of work items; tile_start of the table is not used.
 bool decode_grouped_supports(const GroupTable& tab, int n, int k);

@@ -98,7 +98,7 @@ int fp8_block_gemm_select(int kernel_id);
  * -1 = choose by cost model) and one K-split count
  * (0 = choose, at most 16; more returns FP8GEMM_E_KERNEL).  With FP8GEMM_KERNEL_SKINNY selected the
  * first argument picks the decode kernel instead: 0 = 32-column strips, 1 = 128-column strips whose K
- * splits are added inside the kernel, -1 = by cost.  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
+ * splits are added inside the kernel, 2 = the same with 256-column strips, -1 = by cost.  Benchmarking and test aid; no counterpart in the reference beyond editing its WMMA_* / NUM_WARP_* macros
  * (/root/reference/mn_large.hip:1-8). */
 int fp8_block_gemm_force_config(int tile_variant, int ksplit);
 

@@ -327,6 +327,30 @@ def test_decode_rows_off_the_grid_run_without_a_padded_copy(pkg):
     assert np.array_equal(dc.cpu().numpy().view(np.uint16).reshape(-1), got.reshape(-1))
 
 
+# 256-column strips (tile_variant 2 of the decode family): two 128-column halves per stage, their own b_scale
+# each; strips whose last one ends in its first half / in its second; every row-tile count, rows on and off the
+# 16-byte grid; split and unsplit; results bit-identical to the 128-column strips with the same K split
+DECODE_WIDE_STRIP_CASES = [(32, 7168, 2048, 4), (16, 7168, 2048, 1), (32, 576, 1024, 3), (32, 1200, 2048, 16),
+                           (7, 4608, 7168, 6), (40, 2064, 7168, 8), (63, 256, 128, 1), (1, 18432, 1024, 2),
+                           (24, 16384, 1024, 4), (48, 7168, 2048, 2), (64, 112, 512, 2), (33, 18432, 384, 3)]
+
+
+@pytest.mark.parametrize("m,n,k,ksplit", DECODE_WIDE_STRIP_CASES)
+def test_decode_kernel_with_256_column_strips(pkg, m, n, k, ksplit):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1270 + m + n + k + ksplit, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=2, ksplit=ksplit)
+    assert name == f"decode256_k{ksplit}", name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    narrow, nname = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ksplit)
+    assert nname == f"decode128_k{ksplit}", nname
+    assert np.array_equal(got, narrow), "differs from the 128-column strips"
+    for rep in range(3):
+        again, _ = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=2, ksplit=ksplit)
+        assert np.array_equal(got, again), f"run {rep}: not reproducible"
+
+
 def test_decode_strip_split_that_outgrows_the_mailbox_is_refused(pkg):
     """128 strips x 15 sending splits x 16 KiB of patches do not fit the 16 MiB mailbox: no such plan"""
     m, n, k = 32, 16384, 2048
