@@ -171,9 +171,11 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     // line, extrapolated to its area, would put it 6 % ahead)
     // (a single row of tiles reads every byte of B once and from HBM -- decode weights do not fit the caches --,
     // where a K block takes a quarter longer than the fit to cached operands says: without this factor
-    // 48 x 7168 x 1536 stays unsplit, 9.4 us from HBM against 8.1 us with two splits)
-    const double per_kb =
-        (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * (g.m <= 64 ? 1.25 : 1.0);
+    // 48 x 7168 x 1536 stays unsplit, 9.4 us from HBM against 8.1 us with two splits; the same for two rows of
+    // 64x64 tiles over a large B, which they fetch in 64-byte pieces: 128 x 4096 x 7168 as tile64x64_k2f 22.2 us,
+    // as tile128x128_k7 17.1 us -- while over 1536 x 7168 tile64x64_k5f stays ahead, 11.9 against 12.9 us)
+    const bool streams_b = g.m <= 64 || (variant == TILE_64x64 && g.m <= 128 && (long long)g.n * g.k >= 20000000ll);
+    const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * (streams_b ? 1.25 : 1.0);
     const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     const long items = (long)tiles * ksplit;
     // (two 64x64 workgroups share a CU, but a single row of tiles with B from HBM is fastest with at most one
