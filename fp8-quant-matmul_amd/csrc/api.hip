@@ -114,7 +114,7 @@ inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p)
 
 // conservative = true: every operand copied (an upper bound that does not depend on addresses).
 // keeps_rows = the kernels of the plan take a leading dimension for a and a_scale apart from m
-// (the tile kernels): c then needs no copy on account of m.
+// (the tile kernels and the wide decode strips): c then needs no copy on account of m.
 PadLayout pad_layout(const GemmArgs& g, size_t partial_bytes, bool conservative, bool keeps_rows)
 {
     PadLayout L{};
@@ -292,9 +292,11 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
         if (wide_ok && (by_name ? cfg.force_variant != 0 : cfg.force_variant < 0)) {
             // without the in-kernel reduction (no zeroed mailbox, or workgroup placement not confirmed) only
             // the unsplit form exists.  By name, tile_variant 2 pins the 256-column strips.
-            // Left to the cost model, 256-column strips have to be 7 % ahead: they halve the workgroups of a
-            // split and win where that saves a round (144 strips x 3 splits are 54 workgroups on an XCD's 32 CUs,
-            // 72 x 3 are 27: 18432 x 7168 from HBM 28.6 against 34.6 us), and lose 15 - 40 % on cfg5-sized problems.
+            // Left to the cost model, 256-column strips have to be 7 % ahead in launches of a single round: they
+            // halve the workgroups of a split and win where that saves a round (144 strips x 3 splits are 54
+            // workgroups on an XCD's 32 CUs, 72 x 3 are 27: 18432 x 7168 from HBM 28.6 against 34.6 us), and lose
+            // 15 - 40 % on cfg5-sized problems.  Launches of several rounds stream, and there the wider strips are
+            // ahead throughout (a projection onto a vocabulary with 8 rows, 131072 x 4096: 93.3 against 101.7 us).
             const int hi = cfg.fused_ok ? (nkb < MAX_KSPLIT ? nkb : MAX_KSPLIT) : 1;
             for (int halves = 1; halves <= 2; ++halves) {
                 if (by_name ? halves != (cfg.force_variant == 2 ? 2 : 1) : cfg.force_variant >= 0 && halves == 2)
@@ -302,7 +304,9 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
                 for (int ks = 1; ks <= hi; ++ks) {
                     if (!valid_split(ks) || (forced_ks && ks != forced_ks) || !decode_strip_can_split(g, ks, halves))
                         continue;
-                    const double cst = decode_strip_cost(g, ks, halves) * (halves == 2 && !by_name ? 1.07 : 1.0);
+                    const long per_xcd = (long)(((g.n + 255) / 256 + 7) / 8) * ks;  // workgroups of 256-column strips
+                    const double cst =
+                        decode_strip_cost(g, ks, halves) * (halves == 2 && !by_name && (per_xcd <= 32 || ks > 1) ? 1.07 : 1.0);
                     if (cst < wide_us) {
                         wide_us = cst;
                         wide.ksplit = ks;
@@ -323,6 +327,7 @@ Plan make_plan(const GemmArgs& g, const Config& cfg)
         // (M = 33 ... 63 on the same 12 shapes: 6.8 - 16.9 us against 10.8 - 23.8 us).
         if (!by_name && g.m > 32 && g.m % 16 == 0 && !(g.n >= 6144 && (long long)g.n * g.k >= 28000000ll))
             wide_us = 1e300;
+
         if (!by_name && cfg.force_variant < 0 && cfg.force_ksplit <= 0 && wide_us < 1e300 && cfg.fused_ok)
             return wide;
         if (!by_name && !cfg.fused_ok)
@@ -555,7 +560,8 @@ size_t padded_bytes(const GemmArgs& g, const Plan& p)
     GemmArgs gp = g;
     gp.m = (g.m + 15) & ~15;
     gp.n = (g.n + 15) & ~15;
-    const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK;
+    const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK ||
+                            (p.family == FP8GEMM_KERNEL_SKINNY && p.wide);
     return with_header(pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows).total, plan_uses_header(p));
 }
 
@@ -565,7 +571,8 @@ int run_padded(const GemmArgs& g, const Plan& p, const Workspace& w, hipStream_t
     const int m16 = (g.m + 15) & ~15;
     gp.m = m16;
     gp.n = (g.n + 15) & ~15;
-    const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK;
+    const bool keeps_rows = p.family == FP8GEMM_KERNEL_LARGE || p.family == FP8GEMM_KERNEL_SPLITK ||
+                            (p.family == FP8GEMM_KERNEL_SKINNY && p.wide);
     const PadLayout L = pad_layout(g, plan_workspace_bytes(gp, p), false, keeps_rows);
     if (!L.c) {  // c is written in place: its m rows, while a and a_scale have m16 per k-row
         gp.m = g.m;

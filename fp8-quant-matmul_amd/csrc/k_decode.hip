@@ -471,10 +471,10 @@ __device__ __forceinline__ void decode_body(const DecodeProblem& one, const Grou
 template <int MT, int DS_NS, bool RAGGED, int TILES, int NB>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_strip_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
-                    const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int N, int K,
-                    int strips, int ksplit, int kb_per_split)
+                    const float* __restrict__ b_scale, uint16_t* __restrict__ c, float* mailbox, int M, int lda, int N,
+                    int K, int strips, int ksplit, int kb_per_split)
 {
-    const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
+    const DecodeProblem one{a, b, a_scale, b_scale, c, M, lda};
     decode_body<MT, false, DS_NS, RAGGED, TILES, NB>(one, nullptr, mailbox, N, K, strips, strips, ksplit, kb_per_split);
 }
 
@@ -723,9 +723,10 @@ decode_stream_grouped_kernel(const GroupTable tab, int N, int K, int strips, int
 template <int MT, int DS_NS, int TILES, bool STAGED, int NB>
 __global__ void __launch_bounds__(DS_THREADS)
 decode_stream_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b, const float* __restrict__ a_scale,
-                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, int M, int N, int K, int strips)
+                     const float* __restrict__ b_scale, uint16_t* __restrict__ c, int M, int lda, int N, int K,
+                     int strips)
 {
-    const DecodeProblem one{a, b, a_scale, b_scale, c, M, M};
+    const DecodeProblem one{a, b, a_scale, b_scale, c, M, lda};
     decode_stream_body<MT, DS_NS, TILES, STAGED, NB, false>(one, nullptr, N, K, strips, strips);
 }
 
@@ -761,10 +762,13 @@ inline bool shallow_ring_pays(long workgroups, int kb_per_split) { return workgr
 
 }  // namespace
 
-// any 1 <= m <= 64: a row count off the 16-byte grid runs the kernels that spread A's packed slabs in the LDS
+// any 1 <= m <= 64: a row count off the 16-byte grid runs the kernels that spread A's packed slabs in the LDS;
+// a and a_scale may have more elements per k-row than c has rows (lda: a multiple of 16, at most 64 -- padded
+// copies whose c is written in place)
 bool decode_strip_supports(const GemmArgs& g)
 {
-    return g.m >= 1 && g.m <= 64 && g.n % 16 == 0 && (g.lda == 0 || g.lda == g.m) &&
+    return g.m >= 1 && g.m <= 64 && g.n % 16 == 0 &&
+           (g.lda == 0 || g.lda == g.m || (g.lda > g.m && g.lda <= 64 && g.lda % 16 == 0)) &&
            (reinterpret_cast<uintptr_t>(g.a) % 16 == 0) && (reinterpret_cast<uintptr_t>(g.b) % 16 == 0) &&
            (reinterpret_cast<uintptr_t>(g.a_scale) % 4 == 0) && (reinterpret_cast<uintptr_t>(g.b_scale) % 4 == 0) &&
            (reinterpret_cast<uintptr_t>(g.c) % 8 == 0);
@@ -798,8 +802,10 @@ double decode_strip_cost(const GemmArgs& g, int ksplit, int halves)
     // 19.8 us against 14.0 us with 6 splits for 4608 x 7168)
     const long rounds = ((long)((strips + 7) / 8) * ksplit + 31) / 32;
     const double active = wgs < 256 ? (double)wgs : 256.0;
-    // (a stage of a 256-column strip is twice the bytes for 1.92 times the time)
-    const double per_block = (0.50 + 0.001 * active) * (halves == 2 ? 1.92 : 1.0);
+    // (a stage of a 256-column strip is twice the bytes for 1.92 times the time in a launch of one round, which
+    // lives on latencies, and for 1.8 times in longer unsplit ones, which stream: 256 contiguous bytes come 10 %
+    // faster)
+    const double per_block = (0.50 + 0.001 * active) * (halves == 2 ? (rounds > 1 && ksplit == 1 ? 1.8 : 1.92) : 1.0);
     const double life = 1.0 + kbs * per_block + (ksplit > 1 ? 0.39 * ksplit : 0.0);
     return 2.5 + (double)rounds * life;
 }
@@ -849,10 +855,44 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, int halves, float
     const dim3 grid(8 * ((strips + 7) / 8) * ksplit);
     auto go = [&](auto kern, int lds) -> hipError_t {
         FP8GEMM_ALLOW_LDS(kern, lds);
-        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c, mailbox, g.m, g.n,
-                           g.k, strips, ksplit, kb_per_split);
+        hipLaunchKernelGGL(kern, grid, dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c, mailbox, g.m,
+                           leading_dim(g), g.n, g.k, strips, ksplit, kb_per_split);
         return hipGetLastError();
     };
+    // more 128-column strips than resident workgroups, no K split: one copy stream per workgroup (the streaming
+    // form chooses its strip width itself)
+    const int strips128 = (g.n + DS_BN - 1) / DS_BN;
+    if (ksplit == 1 && strips128 > STREAM_WORKGROUPS && leading_dim(g) % 16 == 0) {
+        const bool staged = reinterpret_cast<uintptr_t>(g.c) % 16 == 0;
+        const int wide_units = (g.n + 2 * DS_BN - 1) / (2 * DS_BN);
+        const bool wide = wide_units >= STREAM_WORKGROUPS;  // 256-column strips while every CU gets one
+        const int units = wide ? wide_units : strips128;
+        auto stream = [&](auto shape, auto tiles_c, auto staged_c) -> hipError_t {
+            constexpr int MT = decltype(shape)::MT, NS = decltype(shape)::NS, NB = decltype(shape)::NB;
+            constexpr int T = decltype(tiles_c)::value;
+            constexpr bool ST = decltype(staged_c)::value;
+            constexpr int lds = DecodeShape<MT, NS, false, NB>::LDS + (ST ? 16 * T * (2 * DS_BN * NB + 16) : 0);
+            static_assert(lds <= 160 * 1024, "ring and staged C exceed the LDS");
+            auto kern = decode_stream_kernel<MT, NS, T, ST, NB>;
+            FP8GEMM_ALLOW_LDS(kern, lds);
+            hipLaunchKernelGGL(kern, dim3(STREAM_WORKGROUPS), dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
+                               g.m, leading_dim(g), g.n, g.k, units);
+            return hipGetLastError();
+        };
+        auto by_staging = [&](auto shape, auto tiles_c) -> hipError_t {
+            return staged ? stream(shape, tiles_c, std::true_type{}) : stream(shape, tiles_c, std::false_type{});
+        };
+        auto by_tiles = [&](auto shape2, auto shape4) -> hipError_t {
+            switch ((g.m + 15) / 16) {
+            case 1: return by_staging(shape2, std::integral_constant<int, 1>{});
+            case 2: return by_staging(shape2, std::integral_constant<int, 2>{});
+            case 3: return by_staging(shape4, std::integral_constant<int, 3>{});
+            default: return by_staging(shape4, std::integral_constant<int, 4>{});
+            }
+        };
+        return wide ? by_tiles(StreamShape<2, STREAM_NS_WIDE, 2>{}, StreamShape<4, STREAM_NS_WIDE, 2>{})
+                    : by_tiles(StreamShape<2, STREAM_NS, 1>{}, StreamShape<4, STREAM_NS4, 1>{});
+    }
     if (halves == 2) {  // 256-column strips: three stages of 32 KB of B
         const int tiles = (g.m + 15) / 16;
         auto wide = [&](auto mt_c, auto ragged_c, auto tiles_c) -> hipError_t {
@@ -868,41 +908,10 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, int halves, float
             default: return wide(std::integral_constant<int, 4>{}, ragged_c, std::integral_constant<int, 4>{});
             }
         };
-        return g.m % 16 != 0 ? by_tiles(std::true_type{}) : by_tiles(std::false_type{});
-    }
-    if (ksplit == 1 && strips > STREAM_WORKGROUPS && g.m % 16 == 0) {  // more units than resident workgroups: one copy stream per workgroup
-        const bool staged = reinterpret_cast<uintptr_t>(g.c) % 16 == 0;
-        const int wide_units = (g.n + 2 * DS_BN - 1) / (2 * DS_BN);
-        const bool wide = wide_units >= STREAM_WORKGROUPS;  // 256-column strips while every CU gets one
-        const int units = wide ? wide_units : strips;
-        auto stream = [&](auto shape, auto tiles_c, auto staged_c) -> hipError_t {
-            constexpr int MT = decltype(shape)::MT, NS = decltype(shape)::NS, NB = decltype(shape)::NB;
-            constexpr int T = decltype(tiles_c)::value;
-            constexpr bool ST = decltype(staged_c)::value;
-            constexpr int lds = DecodeShape<MT, NS, false, NB>::LDS + (ST ? 16 * T * (2 * DS_BN * NB + 16) : 0);
-            static_assert(lds <= 160 * 1024, "ring and staged C exceed the LDS");
-            auto kern = decode_stream_kernel<MT, NS, T, ST, NB>;
-            FP8GEMM_ALLOW_LDS(kern, lds);
-            hipLaunchKernelGGL(kern, dim3(STREAM_WORKGROUPS), dim3(DS_THREADS), lds, s, g.a, g.b, g.a_scale, g.b_scale, g.c,
-                               g.m, g.n, g.k, units);
-            return hipGetLastError();
-        };
-        auto by_staging = [&](auto shape, auto tiles_c) -> hipError_t {
-            return staged ? stream(shape, tiles_c, std::true_type{}) : stream(shape, tiles_c, std::false_type{});
-        };
-        auto by_tiles = [&](auto shape2, auto shape4) -> hipError_t {
-            switch (g.m / 16) {
-            case 1: return by_staging(shape2, std::integral_constant<int, 1>{});
-            case 2: return by_staging(shape2, std::integral_constant<int, 2>{});
-            case 3: return by_staging(shape4, std::integral_constant<int, 3>{});
-            default: return by_staging(shape4, std::integral_constant<int, 4>{});
-            }
-        };
-        return wide ? by_tiles(StreamShape<2, STREAM_NS_WIDE, 2>{}, StreamShape<4, STREAM_NS_WIDE, 2>{})
-                    : by_tiles(StreamShape<2, STREAM_NS, 1>{}, StreamShape<4, STREAM_NS4, 1>{});
+        return leading_dim(g) % 16 != 0 ? by_tiles(std::true_type{}) : by_tiles(std::false_type{});
     }
     const int tiles = (g.m + 15) / 16;
-    if (g.m % 16 != 0) {
+    if (leading_dim(g) % 16 != 0) {
         constexpr int L2 = DecodeShape<2, 6, true>::LDS, L4 = DecodeShape<4, RAGGED4_NS, true>::LDS;
         switch (tiles) {
         case 1: return go(decode_strip_kernel<2, 6, true, 1, 1>, L2);
