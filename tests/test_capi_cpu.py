@@ -234,6 +234,11 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(64, 7168, 7168) == "decode128_k4"
     assert pkg.plan(40, 4608, 7168) == "decode128_k6"      # 36 strips over 8 XCDs: 5 x 6 workgroups on an XCD's 32 CUs
     assert pkg.plan(7, 7168, 2048) == "decode128_k4"       # a decode batch of 7 rows: no padded copy
+    # 256-column strips where they save a round of workgroups on an XCD (144 strips x 3 splits: 54 on 32 CUs;
+    # 72 x 3: 27) and in unsplit launches of several rounds (a projection onto a vocabulary)
+    assert pkg.plan(32, 18432, 7168) == "decode256_k3"
+    assert pkg.plan(8, 131072, 4096) == "decode256_k1"
+    assert pkg.plan(32, 7168, 7168) == "decode128_k4"
     pkg.select(pkg.KERNEL_SKINNY)
     pkg.force_config(-1, 3)
     assert pkg.plan(32, 7168, 2048) == "decode128_k3"      # a pinned K split reaches the decode kernels too
