@@ -38,6 +38,14 @@
 // body runs grouped problems (common N and K, own M <= 64, own operands: the experts of an MoE layer in a
 // decode step), whose strips form one list of work items.
 //
+// Variants of the same body (template arguments): a row count off the 16-byte grid (RAGGED: A's packed K-block
+// slabs are copied whole and spread into padded rows in the LDS); strips of 256 columns (NB = 2: two
+// 128-column halves per stage; 256 contiguous bytes of a k-row come 10 % faster from HBM than 128, at half
+// the workgroups per split); one copy of the K loop per number of row tiles, so that no branch surrounds its
+// LDS operations.  The streaming form (decode_stream_body) is for launches with more strips than the device
+// holds workgroups and no K split: 256 workgroups walk through the strips -- of one problem or of all groups --
+// and the K blocks of all strips of a workgroup form one copy stream.
+//
 // LDS stage: 128 k-rows x 128 B of B (chunk c of row r at position c ^ ((r >> 1) & 7)), 128 x 32 B
 // of A (chunk c at c ^ ((r >> 3) & 1); 64-byte rows: c ^ ((r >> 2) & 3)), the block's a_scale and b_scale values; six stages form a
 // ring, up to five in flight while one is multiplied.  A CU takes in about 50 bytes per clock through
