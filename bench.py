@@ -433,15 +433,15 @@ def main():
                         "parity_pass": par["pass"]})
         return out
 
-    def grouped_decode_report(steps, warmup, experts=64, gn=7168, gk=2048, on_grid=False):
-        """an MoE layer in a decode step: `experts` problems of 1 to 64 rows each (seeded), every expert with
-        its own weights (64 x 14.7 MB: streamed from HBM on every launch).  One grouped call (one launch of
-        the decode kernel on all experts' strips) against one call per expert.  Operands are seeded random
+    def grouped_decode_report(steps, warmup, experts=64, gn=7168, gk=2048, on_grid=False, rows_hi=64):
+        """an MoE layer in a decode step: `experts` problems of 1 to `rows_hi` rows each (seeded), every expert
+        with its own weights (14.7 MB each: streamed from HBM on every launch).  One grouped call (one launch
+        of the decode kernel on the strips of up to 64 experts) against one call per expert.  Operands are seeded random
         bytes and scales generated on the device (parity of the grouped path is the tests' business)."""
         gen = torch.Generator(device="cuda")
         gen.manual_seed(4242)
         rs = __import__("numpy").random.RandomState(4242)
-        ms = [int(v) for v in rs.randint(1, 65, size=experts)]
+        ms = [int(v) for v in rs.randint(1, rows_hi + 1, size=experts)]
         if on_grid:
             ms = [max(16, (v + 15) // 16 * 16) for v in ms]
         bufs = []
@@ -521,6 +521,8 @@ def main():
     if not args.no_shapes:   # 64 experts of 1..64 rows, and the same on the 16-row grid
         grouped_decode = grouped_decode_report(max(20, args.steps), args.warmup)
         grouped_decode["on_grid"] = grouped_decode_report(max(20, args.steps), args.warmup, on_grid=True)
+        # every routed expert of a 256-expert layer live, a few tokens each: four launches of 64 experts
+        grouped_decode["experts256"] = grouped_decode_report(max(20, args.steps), args.warmup, experts=256, rows_hi=8)
     decode_rows = None if args.no_shapes else decode_rows_report(max(20, args.steps), args.warmup)
     host_boundary = None if args.no_shapes else host_boundary_report()
     props = torch.cuda.get_device_properties(0)

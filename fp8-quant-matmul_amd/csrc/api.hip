@@ -25,7 +25,7 @@ std::atomic<int> g_force_ksplit{0};
 std::atomic<int> g_persistent{-1};  // -1 = when tiles outnumber the CUs, 0 = never, 1 = whenever possible
 std::atomic<int> g_fused{-1};       // K splits added inside the GEMM kernel: -1 = by cost, 0 = never, 1 = whenever possible
 thread_local const char* t_last_kernel = "none";
-thread_local char t_name_buf[64];
+thread_local char t_name_buf[96];
 
 // what decides a plan besides the shape
 struct Config {
@@ -1039,9 +1039,13 @@ static int run_grouped(int groups, const void* const* a, const void* const* b, c
         return FP8GEMM_OK;
     if (!a || !b || !a_scale || !b_scale || !c || !m)
         return FP8GEMM_E_NULLPTR;
+    // Groups of at most 64 rows (an MoE layer in a decode step) go to the decode kernel, which streams
+    // every group's B once in whole lines; taller groups to the persistent tile kernel.  A pinned tile
+    // shape sends everything to the tile kernel.
+    auto is_small = [&](int g) { return m[g] <= 64 && cfg.force_variant < 0; };
     // every problem is validated before anything is launched
     long long m_total = 0;
-    int live = 0;
+    int count[2] = {0, 0};  // small, tall
     for (int g = 0; g < groups; ++g) {
         if (m[g] < 0)
             return FP8GEMM_E_SHAPE;
@@ -1051,48 +1055,59 @@ static int run_grouped(int groups, const void* const* a, const void* const* b, c
         if (v != FP8GEMM_OK)
             return v;
         m_total += m[g];
-        ++live;
+        ++count[is_small(g) ? 0 : 1];
     }
-    if (live == 0)
+    if (count[0] + count[1] == 0)
         return FP8GEMM_OK;
     static_assert(GroupTable::MAX_GROUPS == FP8GEMM_MAX_GROUPS, "table size mirrors the ABI constant");
-    if (live <= GroupTable::MAX_GROUPS && cfg.selected == FP8GEMM_KERNEL_AUTO && m_total <= 0x7FFFFFFFll) {
-        // Groups of at most 64 rows (an MoE layer in a decode step) go to the decode kernel, which streams
-        // every group's B once in whole lines; taller groups to the persistent tile kernel.  A pinned tile
-        // shape sends everything to the tile kernel.
-        GroupTable small, tall;
-        small.groups = tall.groups = 0;
-        for (int g = 0; g < groups; ++g) {
-            if (m[g] == 0)
-                continue;
-            GroupTable& tab = (m[g] <= 64 && cfg.force_variant < 0) ? small : tall;
-            const int t = tab.groups++;
-            tab.a[t] = static_cast<const uint8_t*>(a[g]);
-            tab.b[t] = static_cast<const uint8_t*>(b[g]);
-            tab.a_scale[t] = a_scale[g];
-            tab.b_scale[t] = b_scale[g];
-            tab.c[t] = static_cast<uint16_t*>(c[g]);
-            tab.m[t] = m[g];
-            tab.lda[t] = m[g];
-        }
+    if (cfg.selected == FP8GEMM_KERNEL_AUTO && m_total <= 0x7FFFFFFFll) {
+        // One launch holds MAX_GROUPS problems (the table travels in the kernel arguments): more of a kind run
+        // as the fewest launches that hold them, of equal size, one after the other on the stream.
         int rc = FP8GEMM_OK;
         char first_name[sizeof(t_name_buf)] = "";
-        if (small.groups > 0) {
-            rc = run_grouped_table(small, n, k, true, s, cfg, explicit_ws);
-            if (rc == FP8GEMM_OK && tall.groups > 0)
+        for (int kind = 0; kind < 2 && rc == FP8GEMM_OK; ++kind) {
+            if (count[kind] == 0)
+                continue;
+            const int launches = (count[kind] + GroupTable::MAX_GROUPS - 1) / GroupTable::MAX_GROUPS;
+            const int per_launch = (count[kind] + launches - 1) / launches;
+            GroupTable tab;
+            tab.groups = 0;
+            int seen = 0;
+            for (int g = 0; g < groups && rc == FP8GEMM_OK; ++g) {
+                if (m[g] == 0 || is_small(g) != (kind == 0))
+                    continue;
+                const int t = tab.groups++;
+                tab.a[t] = static_cast<const uint8_t*>(a[g]);
+                tab.b[t] = static_cast<const uint8_t*>(b[g]);
+                tab.a_scale[t] = a_scale[g];
+                tab.b_scale[t] = b_scale[g];
+                tab.c[t] = static_cast<uint16_t*>(c[g]);
+                tab.m[t] = m[g];
+                tab.lda[t] = m[g];
+                ++seen;
+                if (tab.groups == per_launch || seen == count[kind]) {
+                    rc = run_grouped_table(tab, n, k, kind == 0, s, cfg, explicit_ws);
+                    tab.groups = 0;
+                }
+            }
+            if (rc != FP8GEMM_OK)
+                break;
+            if (launches > 1) {  // the last launch's name and how many there were
+                char many[sizeof(t_name_buf)];
+                snprintf(many, sizeof(many), "%.88sx%d", t_name_buf, launches);
+                snprintf(t_name_buf, sizeof(t_name_buf), "%s", many);
+            }
+            if (kind == 0 && count[1] > 0)
                 snprintf(first_name, sizeof(first_name), "%s", t_name_buf);
-        }
-        if (rc == FP8GEMM_OK && tall.groups > 0) {
-            rc = run_grouped_table(tall, n, k, false, s, cfg, explicit_ws);
-            if (rc == FP8GEMM_OK && first_name[0]) {  // both kernels ran: name both
+            if (kind == 1 && first_name[0]) {  // both kernels ran: name both
                 char both[sizeof(t_name_buf)];
-                snprintf(both, sizeof(both), "%.28s+%.30s", first_name, t_name_buf);
+                snprintf(both, sizeof(both), "%.46s+%.46s", first_name, t_name_buf);
                 snprintf(t_name_buf, sizeof(t_name_buf), "%s", both);
             }
         }
         if (rc != GROUPED_NOT_APPLICABLE)
             return rc;
-        // (a decode launch that already ran is simply run again below: same inputs, same outputs)
+        // (launches that already ran are simply run again below: same inputs, same outputs)
     }
     for (int g = 0; g < groups; ++g) {
         if (m[g] == 0)

@@ -135,8 +135,9 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * once, the K range split and added inside the kernel as for a single problem; row counts off the 16-row
  * grid as they are, without copies, except in launches large enough for the streaming form -- 256 or more
  * strips of 256 columns over all groups --, which runs on padded copies of A and a_scale); a call that mixes
- * both kinds launches each kernel once.  More groups than FP8GEMM_MAX_GROUPS fall back to one call
- * of fp8_block_gemm_stream per group, with the same results.  Each C[g] is bit-identical to
+ * both kinds launches each kernel once.  A launch holds FP8GEMM_MAX_GROUPS problems; more of a kind run as
+ * the fewest launches that hold them, of equal size, one after the other on the stream ("...groupedGxL":
+ * L launches, the last of G groups).  Each C[g] is bit-identical to
  * what fp8_block_gemm_stream gives for that problem with the same tile shape (decode kernel: with the
  * same K split).  No counterpart in the
  * reference, which launches one problem at a time (/root/reference/check.cu:106-114). */

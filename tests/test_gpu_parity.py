@@ -858,14 +858,29 @@ def test_grouped_gemm_with_a_tile_shape_that_has_no_grouped_form(pkg):
         _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
 
 
-def test_grouped_gemm_takes_more_groups_than_one_launch_holds(pkg):
-    """70 groups (one launch holds 64): the groups run one by one, ragged ones on padded copies"""
-    ms, n, k = [16 + (g % 3) for g in range(70)], 64, 128
-    host, dev, outs, name = _grouped_case(pkg, ms, n, k, -1, 8300)
-    assert "_grouped" not in name, name
+@pytest.mark.parametrize("ms,n,k,expect", [
+    ([16 + (g % 3) for g in range(70)], 64, 128, "decode128_k1_grouped35x2"),
+    ([1 + (5 * g) % 64 for g in range(130)], 512, 384, "_grouped42x3"),                       # 44 + 44 + 42
+    ([0, 0] + [16] * 64 + [0], 256, 256, "_grouped64"),                                       # 64 live ones: one launch
+    ([(8 if g % 2 else 80 + g) for g in range(150)], 256, 256, "_grouped37x2+"),              # 75 small, 75 tall
+])
+def test_grouped_gemm_takes_more_groups_than_one_launch_holds(pkg, ms, n, k, expect):
+    """more groups than a launch holds (64) run as the fewest launches of equal size, every group as in a
+    call of its own"""
+    host, dev, outs, name = _grouped_case(pkg, ms, n, k, -1, 8300 + len(ms))
+    assert expect in name, name
+    if "+" in expect:
+        assert name.endswith("_grouped37x2"), name
     for g, m in enumerate(ms):
+        got = outs[g].cpu().numpy().view(np.uint16)
+        assert (got[m:] == 0x7FC1).all(), f"group {g}: rows beyond m written"
+        if m == 0:
+            continue
         a, b, sa, sb = host[g]
-        _assert_close(outs[g].cpu().numpy().view(np.uint16), oracle.ref_gemm(a, b, sa, sb, m, n, k), f"group {g}")
+        # buffers made for 16 rows and read with m < 16 per k-row: the first k * m values, as the kernel sees them
+        a_seen = np.ascontiguousarray(a.reshape(-1)[:k * m].reshape(k, m))
+        sa_seen = np.ascontiguousarray(sa.reshape(-1)[:(k // 128) * m].reshape(k // 128, m))
+        _assert_close(got[:m], oracle.ref_gemm(a_seen, b, sa_seen, sb, m, n, k), f"group {g}")
     pkg.release()
 
 
