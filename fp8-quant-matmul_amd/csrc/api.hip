@@ -175,18 +175,29 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     // 64x64 tiles over a large B, which they fetch in 64-byte pieces: 128 x 4096 x 7168 as tile64x64_k2f 22.2 us,
     // as tile128x128_k7 17.1 us -- while over 1536 x 7168 tile64x64_k5f stays ahead, 11.9 against 12.9 us)
     const bool streams_b = g.m <= 64 || (variant == TILE_64x64 && g.m <= 128 && (long long)g.n * g.k >= 20000000ll);
-    const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * (streams_b ? 1.25 : 1.0);
-    const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     const long items = (long)tiles * ksplit;
+    // (a problem of at most 64 tiles of 64x64: a K block takes 0.265 us whether 4 or 64 tiles run -- M, N = 96 ... 512
+    // with K = 1536 ... 8192 -- where the fit, made on launches of several rounds, says 0.34, and the hand-over of
+    // the splits inside the kernel starts 0.3 us earlier.  Problems of 96 ... 256 such tiles measure as the fit
+    // says, or slower.)
+    const bool light = variant == TILE_64x64 && !streams_b && tiles <= 64;
+    const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * (streams_b ? 1.25 : 1.0) *
+                          (light ? 0.8 : 1.0);
+    const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
     // (two 64x64 workgroups share a CU, but a single row of tiles with B from HBM is fastest with at most one
     // workgroup per CU: M = 48, 64 on 12 shapes, the split that keeps tiles x splits within 256 is the best
     // measured or within 2 % of it)
     const long rounds = (items + NUM_CU - 1) / NUM_CU;
     double cost = 1.79 + rounds * per_item;
     if (ksplit > 1 && fused)  // the last split of a tile waits for the others' accumulators and reads them
-        cost += 1.8 + 0.35 * (ksplit - 1) * (double)(bm * bn) / 4096.0;
-    else if (ksplit > 1)  // second launch + partial write and read-back
+        cost += (light ? 1.5 : 1.8) + 0.35 * (ksplit - 1) * (double)(bm * bn) / 4096.0;
+    else if (ksplit > 1) {  // second launch + partial write and read-back
         cost += 2.86 + (double)g.m * g.n * ksplit * 8.0 / 7.38e6;
+        // (a GEMM kernel shorter than a launch takes cannot hide the reduction's launch behind it: two such kernels
+        // take 9 - 9.5 us back to back whatever the split, 112 x 96 x 1536 ... 256 x 256 x 7168)
+        const double first = rounds * per_item;
+        cost += first < 4.5 ? 4.5 - first : 0.0;
+    }
     return cost;
 }
 

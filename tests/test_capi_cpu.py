@@ -218,6 +218,12 @@ def test_dispatcher_plans(pkg):
     assert pkg.workspace_bytes(33, 100, 128) >= 128 * 48 + 128 * 112 + 48 * 4 + 48 * 112 * 2
     ks = int(pkg.plan(2048, 576, 7168).split("_k")[1].rstrip("f"))
     assert ks > 1                                          # few tiles, long K: split
+    # a handful of 64x64 tiles: one launch (unsplit, or the splits added inside the kernel), not a split of
+    # every few K blocks with a reduction kernel behind it
+    assert pkg.plan(112, 96, 1536) == "tile64x64_k1"
+    assert pkg.plan(128, 128, 7168) == "tile64x64_k7f"
+    assert pkg.plan(256, 256, 3072) == "tile64x64_k4f"
+    assert pkg.plan(1536, 64, 2304) == "tile64x64_k3f"
     # decode shapes (M <= 32): 128-column strips with the K range split so that one round of workgroups
     # (at most 256) streams B, the splits added inside the kernel
     assert pkg.plan(32, 7168, 2048) == "decode128_k4"      # 56 strips x 4
