@@ -175,7 +175,10 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     // 64x64 tiles over a large B, which they fetch in 64-byte pieces: 128 x 4096 x 7168 as tile64x64_k2f 22.2 us,
     // as tile128x128_k7 17.1 us -- while over 1536 x 7168 tile64x64_k5f stays ahead, 11.9 against 12.9 us)
     const bool streams_b = g.m <= 64 || (variant == TILE_64x64 && g.m <= 128 && (long long)g.n * g.k >= 20000000ll);
-    const long items = (long)tiles * ksplit;
+    // (with the splits added inside the kernel the grid holds a multiple of 8 tiles, so that the splits of a tile
+    // share an XCD: the workgroups beyond the tiles exit at once but take their turn -- 85 tiles x 3 splits are
+    // 264 workgroups, and the last of them start when a CU frees up: 20.2 us against 13.9 us with two splits)
+    const long items = (long)(ksplit > 1 && fused ? (tiles + 7) / 8 * 8 : tiles) * ksplit;
     // (a problem of at most 64 tiles of 64x64: a K block takes 0.265 us whether 4 or 64 tiles run -- M, N = 96 ... 512
     // with K = 1536 ... 8192 -- where the fit, made on launches of several rounds, says 0.34, and the hand-over of
     // the splits inside the kernel starts 0.3 us earlier.  Problems of 96 ... 256 such tiles measure as the fit

@@ -224,6 +224,10 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(128, 128, 7168) == "tile64x64_k7f"
     assert pkg.plan(256, 256, 3072) == "tile64x64_k4f"
     assert pkg.plan(1536, 64, 2304) == "tile64x64_k3f"
+    # 85 tiles x 3 splits added inside the kernel would be 88 x 3 workgroups (the splits of a tile share an XCD):
+    # more than one round
+    assert pkg.plan(2144, 608, 3072) == "tile128x128_k2f"
+    assert pkg.plan(2048, 576, 3072) == "tile128x128_k3f"  # 80 tiles x 3: one round
     # decode shapes (M <= 32): 128-column strips with the K range split so that one round of workgroups
     # (at most 256) streams B, the splits added inside the kernel
     assert pkg.plan(32, 7168, 2048) == "decode128_k4"      # 56 strips x 4
