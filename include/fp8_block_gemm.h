@@ -135,7 +135,9 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * once, the K range split and added inside the kernel as for a single problem; row counts off the 16-row
  * grid as they are, without copies, except in launches large enough for the streaming form -- 256 or more
  * strips of 256 columns over all groups --, which runs on padded copies of A and a_scale); a call that mixes
- * both kinds launches each kernel once.  A launch holds FP8GEMM_MAX_GROUPS problems; more of a kind run as
+ * both kinds launches each kernel once, unless the small groups are few beside the taller ones (at most a third
+ * as many), which then join the tile launch.  Taller groups of up to 256 rows take the 256x256 tile (one row of
+ * tiles each: every group's B is streamed once, in pieces of 256 bytes).  A launch holds FP8GEMM_MAX_GROUPS problems; more of a kind run as
  * the fewest launches that hold them, of equal size, one after the other on the stream ("...groupedGxL":
  * L launches, the last of G groups).  Each C[g] is bit-identical to
  * what fp8_block_gemm_stream gives for that problem with the same tile shape (decode kernel: with the

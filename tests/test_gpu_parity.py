@@ -946,6 +946,39 @@ def test_grouped_decode_groups_off_the_16_byte_grid_and_mixed_with_tall_groups(p
     pkg.release()
 
 
+@pytest.mark.parametrize("ms,n,k,expect", [
+    ([16, 160, 144, 208, 96, 128, 272], 512, 256, "tile256x256_k1_grouped7"),          # one small group rides along
+    ([5, 161, 144, 200, 96, 130, 272, 64], 320, 384, "padded_tile256x256_k1_grouped8"),   # ragged: all on padded copies
+    ([5, 160, 144, 208, 96, 128, 272], 512, 256, "_grouped1+tile256x256_k1_grouped6"),            # tall ones on the grid
+    ([16, 32, 160, 144, 208], 512, 256, "+tile256x256_k1_grouped3"),                     # too many small ones to fold
+    ([300, 700, 512, 160], 768, 256, "_grouped4"),                                      # taller groups: the cost model's shape
+])
+def test_grouped_tile_launch_of_groups_of_one_tile_and_small_groups_riding_along(pkg, ms, n, k, expect):
+    """groups of up to 256 rows take the 256x256 tile (one tile row each, B streamed once); a few groups of at
+    most 64 rows beside many taller ones join the tile launch unless that alone would force padded copies"""
+    import torch
+    st = torch.cuda.current_stream().cuda_stream
+    host, dev, outs = [], [], []
+    for g, m in enumerate(ms):
+        a, b, sa, sb = oracle.make_inputs(m, n, k, 9700 + 13 * g + n)
+        host.append((a, b, sa, sb))
+        dev.append(_dev(a, b, sa, sb))
+        outs.append(torch.full((m + 16, n), 0x7FC1, dtype=torch.int32, device="cuda").to(torch.int16))
+    _say(f"[gpu case] grouped, groups of one tile ms={ms} n={n} k={k}")
+    pkg.gemm_grouped([d[0] for d in dev], [d[1] for d in dev], [d[2] for d in dev], [d[3] for d in dev],
+                     outs, ms, n, k, st)
+    torch.cuda.synchronize()
+    name = pkg.last_kernel()
+    assert name.endswith(expect) and (expect[0] in "+_" or name == expect), name
+    for g, m in enumerate(ms):
+        got = outs[g].cpu().numpy().view(np.uint16)
+        assert (got[m:] == 0x7FC1).all(), f"group {g}: rows beyond m written"
+        a, b, sa, sb = host[g]
+        _assert_close(got[:m], oracle.ref_gemm(a, b, sa, sb, m, n, k), f"{name} group {g}")
+        _assert_every_element(got[:m], a, b, sa, sb, m, n, k, f"{name} group {g}")
+    pkg.release()
+
+
 def test_seeded_sweep_of_shapes_and_plans(pkg):
     """forty pseudo-random (shape, tile, K split, persistence) combinations against the oracle"""
     rs = np.random.RandomState(20241125)
