@@ -163,7 +163,7 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
 {
     int bm, bn;
     tile_variant_dims(variant, &bm, &bn);
-    const int tiles = ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
+    const long tiles = (long)((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn);
     const int nkb = g.k / 128;
     const int kbs = (nkb + ksplit - 1) / ksplit;
     const double area = (double)bm * bn / 65536.0;
@@ -178,7 +178,7 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     // (with the splits added inside the kernel the grid holds a multiple of 8 tiles, so that the splits of a tile
     // share an XCD: the workgroups beyond the tiles exit at once but take their turn -- 85 tiles x 3 splits are
     // 264 workgroups, and the last of them start when a CU frees up: 20.2 us against 13.9 us with two splits)
-    const long items = (long)(ksplit > 1 && fused ? (tiles + 7) / 8 * 8 : tiles) * ksplit;
+    const long items = (ksplit > 1 && fused ? (tiles + 7) / 8 * 8 : tiles) * ksplit;
     // (a problem of at most 64 tiles of 64x64: a K block takes 0.265 us whether 4 or 64 tiles run -- M, N = 96 ... 512
     // with K = 1536 ... 8192 -- where the fit, made on launches of several rounds, says 0.34, and the hand-over of
     // the splits inside the kernel starts 0.3 us earlier.  Problems of 96 ... 256 such tiles measure as the fit
@@ -727,8 +727,22 @@ int scratch_for_current_device(void** out)
     return FP8GEMM_OK;
 }
 
-// tile shape for a grouped launch: what the cost model picks for the stacked problem, among the
-// shapes that have a grouped form, without a K split; -1 when none can take the table
+// the tiles of a grouped launch: every group starts a tile row of its own
+long grouped_tiles(const GroupTable& tab, int n, int variant)
+{
+    int bm, bn;
+    tile_variant_dims(variant, &bm, &bn);
+    long rows = 0;
+    for (int g = 0; g < tab.groups; ++g)
+        rows += (tab.m[g] + bm - 1) / bm;
+    return rows * ((n + bn - 1) / bn);
+}
+
+// tile shape for a grouped launch: what the cost model picks for the stacked problem, among the shapes that
+// have a grouped form, without a K split; -1 when none can take the table.  (Priced with the launch's own tile
+// count -- every group starts a tile row -- the model turns to smaller tiles, which waste fewer rows and measure
+// 17 - 40 % slower: a grouped launch moves more bytes per flop than the single problems the model was fitted
+// on, and the large tiles move the fewest.)
 int grouped_variant(const GroupTable& tab, int n, int k, const Config& cfg)
 {
     long long m_total = 0;
@@ -746,7 +760,9 @@ int grouped_variant(const GroupTable& tab, int n, int k, const Config& cfg)
     int single_tile_groups = 0;
     for (int g = 0; g < tab.groups; ++g)
         single_tile_groups += tab.m[g] <= 256 ? 1 : 0;
-    if (fv < 0 && 4 * single_tile_groups >= 3 * tab.groups && tile_grouped_supports(tab, n, k, TILE_256x256))
+    // (with enough tiles for three quarters of the CUs; fewer are left to the cost model's smaller shapes)
+    if (fv < 0 && 4 * single_tile_groups >= 3 * tab.groups && grouped_tiles(tab, n, TILE_256x256) >= 3 * NUM_CU / 4 &&
+        tile_grouped_supports(tab, n, k, TILE_256x256))
         return TILE_256x256;
     const GemmArgs stacked{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], (int)m_total, n, k};
     for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
@@ -879,6 +895,11 @@ int run_grouped_table(const GroupTable& tab, int n, int k, bool decode, hipStrea
     if (!decode) {
         variant = grouped_variant(pt, n16, k, cfg);
         if (variant < 0)
+            return GROUPED_NOT_APPLICABLE;
+        // A launch that leaves a third of the CUs without a tile while each tile walks a long K range: single
+        // problems split K (one group of 200 x 4096 x 7168: 19 us against 52 us, two: 42 against 56 us; four groups
+        // of 1536 x 7168: level; with K = 2048 one group 13.4 against 15.6 us, two 26 against 19 us).
+        if (cfg.force_variant < 0 && tab.groups <= 8 && k >= 2048 && grouped_tiles(pt, n16, variant) < 160)
             return GROUPED_NOT_APPLICABLE;
     }
     hipError_t e = hipSuccess;
@@ -1125,6 +1146,12 @@ static int run_grouped(int groups, const void* const* a, const void* const* b, c
                 ++seen;
                 if (tab.groups == per_launch || seen == count[kind]) {
                     rc = run_grouped_table(tab, n, k, kind == 0, s, cfg, explicit_ws);
+                    if (rc == GROUPED_NOT_APPLICABLE) {  // these groups one by one
+                        rc = FP8GEMM_OK;
+                        for (int t = 0; t < tab.groups && rc == FP8GEMM_OK; ++t)
+                            rc = run(tab.a[t], tab.b[t], tab.a_scale[t], tab.b_scale[t], tab.c[t], tab.m[t], n, k, s, cfg,
+                                     explicit_ws);
+                    }
                     tab.groups = 0;
                 }
             }
@@ -1143,9 +1170,7 @@ static int run_grouped(int groups, const void* const* a, const void* const* b, c
                 snprintf(t_name_buf, sizeof(t_name_buf), "%s", both);
             }
         }
-        if (rc != GROUPED_NOT_APPLICABLE)
-            return rc;
-        // (launches that already ran are simply run again below: same inputs, same outputs)
+        return rc;
     }
     for (int g = 0; g < groups; ++g) {
         if (m[g] == 0)

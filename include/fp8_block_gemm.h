@@ -137,7 +137,9 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * strips of 256 columns over all groups --, which runs on padded copies of A and a_scale); a call that mixes
  * both kinds launches each kernel once, unless the small groups are few beside the taller ones (at most a third
  * as many), which then join the tile launch.  Taller groups of up to 256 rows take the 256x256 tile (one row of
- * tiles each: every group's B is streamed once, in pieces of 256 bytes).  A launch holds FP8GEMM_MAX_GROUPS problems; more of a kind run as
+ * tiles each: every group's B is streamed once, in pieces of 256 bytes).  A tile launch of at most 8 groups that
+ * would leave more than a third of the CUs without a tile while K >= 2048 is not made: those groups run one by
+ * one, where the dispatcher splits K.  A launch holds FP8GEMM_MAX_GROUPS problems; more of a kind run as
  * the fewest launches that hold them, of equal size, one after the other on the stream ("...groupedGxL":
  * L launches, the last of G groups).  Each C[g] is bit-identical to
  * what fp8_block_gemm_stream gives for that problem with the same tile shape (decode kernel: with the
