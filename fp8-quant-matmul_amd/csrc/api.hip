@@ -738,11 +738,29 @@ long grouped_tiles(const GroupTable& tab, int n, int variant)
     return rows * ((n + bn - 1) / bn);
 }
 
-// tile shape for a grouped launch: what the cost model picks for the stacked problem, among the shapes that
-// have a grouped form, without a K split; -1 when none can take the table.  (Priced with the launch's own tile
-// count -- every group starts a tile row -- the model turns to smaller tiles, which waste fewer rows and measure
-// 17 - 40 % slower: a grouped launch moves more bytes per flop than the single problems the model was fitted
-// on, and the large tiles move the fewest.)
+// Estimated run time of a grouped tile launch in microseconds: tile_cost's form -- launch + rounds of 256
+// workgroups x (fill + K blocks + store) -- on the launch's own tile count, with a K block priced for operands
+// that come from HBM: every group brings its own B, and a tile row of a group reads all of it, so the launch
+// moves more bytes per flop than the single problems tile_cost was fitted on, the more the smaller the tile.
+// Factors on the K block from 25 launches (1 ... 64 groups of 65 ... 3000 rows, N = 1536 ... 7168, K = 2048 and
+// 7168, every tile shape pinned): 1.12 for 256x256, 1.5 for 256x192 and 256x128, 1.7 for 128x192 and 128x128 --
+// e.g. 8 groups of 300 ... 3000 rows, 4608 x 7168: 498 / 610 / 680 / 775 / 893 us estimated for 256x256 / 256x192 /
+// 256x128 / 128x192 / 128x128, 515 / 615 / 727 / 875 / 1042 us measured; 4 groups of 65 ... 256 rows, 7168 x 2048:
+// 35 / 34 / 26 / 46 / 37 us estimated, 32 / 33 / 25 / 42 / 36 us measured.
+double grouped_tile_cost(const GroupTable& tab, int n, int k, int variant)
+{
+    int bm, bn;
+    tile_variant_dims(variant, &bm, &bn);
+    const double area = (double)bm * bn / 65536.0;
+    const double from_hbm = variant == TILE_256x256 ? 1.12 : bm == 256 ? 1.5 : 1.7;
+    const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * from_hbm;
+    const double per_item = 0.95 + 4.38 * area + (k / 128) * per_kb;
+    const long rounds = (grouped_tiles(tab, n, variant) + NUM_CU - 1) / NUM_CU;
+    return 1.79 + rounds * per_item;
+}
+
+// tile shape for a grouped launch: the cheapest by grouped_tile_cost among the shapes that have a grouped form
+// (no K split); -1 when none can take the table
 int grouped_variant(const GroupTable& tab, int n, int k, const Config& cfg)
 {
     long long m_total = 0;
@@ -753,22 +771,12 @@ int grouped_variant(const GroupTable& tab, int n, int k, const Config& cfg)
     int best_v = -1;
     double best = 1e300;
     const int fv = cfg.force_variant;
-    // Groups of up to 256 rows stream their B once whatever the tile, and the launch runs at the rate B comes in:
-    // the 256x256 tile asks for it in pieces of 256 bytes and is 20 - 40 % ahead of every other shape, also
-    // where half its rows are empty (30 groups of 160 rows, N = 7168, K = 2048: 152 us against 205 us for
-    // 256x192, 270 us for 128x128, which reads B twice; 64 groups of 65 ... 300 rows, N = 1536: 84 against 119 us).
-    int single_tile_groups = 0;
-    for (int g = 0; g < tab.groups; ++g)
-        single_tile_groups += tab.m[g] <= 256 ? 1 : 0;
-    // (with enough tiles for three quarters of the CUs; fewer are left to the cost model's smaller shapes)
-    if (fv < 0 && 4 * single_tile_groups >= 3 * tab.groups && grouped_tiles(tab, n, TILE_256x256) >= 3 * NUM_CU / 4 &&
-        tile_grouped_supports(tab, n, k, TILE_256x256))
-        return TILE_256x256;
-    const GemmArgs stacked{tab.a[0], tab.b[0], tab.a_scale[0], tab.b_scale[0], tab.c[0], (int)m_total, n, k};
     for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
         if ((fv >= 0 && v != fv) || !tile_grouped_supports(tab, n, k, v))
             continue;
-        const double cst = tile_cost(stacked, v, 1);
+        if (fv < 0 && persistent_only(v) && !persistent_only_auto(v))
+            continue;
+        const double cst = grouped_tile_cost(tab, n, k, v);
         if (cst < best) {
             best = cst;
             best_v = v;

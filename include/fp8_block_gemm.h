@@ -136,8 +136,9 @@ int fp8_block_gemm_set_fused_reduction(int mode);
  * grid as they are, without copies, except in launches large enough for the streaming form -- 256 or more
  * strips of 256 columns over all groups --, which runs on padded copies of A and a_scale); a call that mixes
  * both kinds launches each kernel once, unless the small groups are few beside the taller ones (at most a third
- * as many), which then join the tile launch.  Taller groups of up to 256 rows take the 256x256 tile (one row of
- * tiles each: every group's B is streamed once, in pieces of 256 bytes).  A tile launch of at most 8 groups that
+ * as many), which then join the tile launch.  The tile shape of a grouped launch comes from a cost model of its
+ * own (its own tile count, K blocks priced for operands from HBM: mostly the 256x256 tile, which streams a
+ * group's B once per 256 rows in pieces of 256 bytes).  A tile launch of at most 8 groups that
  * would leave more than a third of the CUs without a tile while K >= 2048 is not made: those groups run one by
  * one, where the dispatcher splits K.  A launch holds FP8GEMM_MAX_GROUPS problems; more of a kind run as
  * the fewest launches that hold them, of equal size, one after the other on the stream ("...groupedGxL":
