@@ -172,9 +172,11 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     // (a single row of tiles reads every byte of B once and from HBM -- decode weights do not fit the caches --,
     // where a K block takes a quarter longer than the fit to cached operands says: without this factor
     // 48 x 7168 x 1536 stays unsplit, 9.4 us from HBM against 8.1 us with two splits; the same for two rows of
-    // 64x64 tiles over a large B, which they fetch in 64-byte pieces: 128 x 4096 x 7168 as tile64x64_k2f 22.2 us,
-    // as tile128x128_k7 17.1 us -- while over 1536 x 7168 tile64x64_k5f stays ahead, 11.9 against 12.9 us)
-    const bool streams_b = g.m <= 64 || (variant == TILE_64x64 && g.m <= 128 && (long long)g.n * g.k >= 20000000ll);
+    // to four rows of 64x64 tiles over a B of 16 MB or more, which they fetch in 64-byte pieces: 128 x 4096 x 7168
+    // as tile64x64_k2f 22.2 us, as tile128x128_k7 17.1 us; 176 x 4608 x 4096 as tile64x64_k1 21.2 us from HBM and
+    // 12.8 us with B in the Infinity Cache, as tile128x128_k3f 16.6 and 15.9 us -- while over 1536 x 7168
+    // tile64x64_k5f stays ahead, 11.9 against 12.9 us)
+    const bool streams_b = g.m <= 64 || (variant == TILE_64x64 && g.m <= 256 && (long long)g.n * g.k >= 16000000ll);
     // (with the splits added inside the kernel the grid holds a multiple of 8 tiles, so that the splits of a tile
     // share an XCD: the workgroups beyond the tiles exit at once but take their turn -- 85 tiles x 3 splits are
     // 264 workgroups, and the last of them start when a CU frees up: 20.2 us against 13.9 us with two splits)
