@@ -1128,6 +1128,10 @@ static int run_grouped(int groups, const void* const* a, const void* const* b, c
     }
     if (count[0] + count[1] == 0)
         return FP8GEMM_OK;
+    if (count[0] + count[1] == 1 && cfg.force_variant < 0)  // one problem: the dispatcher for single problems
+        for (int g = 0; g < groups; ++g)
+            if (m[g] > 0)
+                return run(a[g], b[g], a_scale[g], b_scale[g], c[g], m[g], n, k, s, cfg, explicit_ws);
     static_assert(GroupTable::MAX_GROUPS == FP8GEMM_MAX_GROUPS, "table size mirrors the ABI constant");
     if (cfg.selected == FP8GEMM_KERNEL_AUTO && m_total <= 0x7FFFFFFFll) {
         // One launch holds MAX_GROUPS problems (the table travels in the kernel arguments): more of a kind run

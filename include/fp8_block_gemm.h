@@ -125,7 +125,8 @@ int fp8_block_gemm_set_fused_reduction(int mode);
 /* Grouped GEMM: `groups` independent problems with the same n and k and their own m[g]
  * (ragged M, e.g. the experts of one MoE layer), C[g] = A[g] . B[g]^T with the layouts above.
  * a, b, a_scale, b_scale, c and m are HOST arrays of `groups` entries; the pointers they hold
- * are device pointers.  Groups with m[g] == 0 are skipped.  Up to FP8GEMM_MAX_GROUPS problems
+ * are device pointers.  Groups with m[g] == 0 are skipped; a call with one group left is
+ * fp8_block_gemm_stream on that group.  Up to FP8GEMM_MAX_GROUPS problems
  * run as ONE launch of the persistent tile kernel (their tiles form one list that 256
  * workgroups walk through): as they are when every m[g] and n are multiples of 16 and the
  * operands 16-byte aligned, else on zero-padded copies in the workspace made by one batched copy
