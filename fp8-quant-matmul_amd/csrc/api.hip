@@ -269,7 +269,48 @@ void decide_fused(const GemmArgs& g, Plan& p, const Config& cfg)
     p.fused = tile_plan_fused(g, p.variant, p.ksplit, cfg);
 }
 
+Plan compute_plan(const GemmArgs& g, const Config& cfg);
+
+// The plan of a problem depends on its sizes, on the low address bits of its operands and on the switches: a
+// serving loop asks for the same few again and again, and working one out costs a microsecond or two of host
+// time (three are worked out per call), which is what a launch-bound decode loop runs on.  Each thread keeps the
+// last plans it worked out, 64 slots indexed by a hash of the sizes.
+struct PlanKey {
+    int m, n, k, lda;
+    uint32_t low_bits;  // 6 low address bits of a, b, a_scale, b_scale and c
+    int selected, force_variant, force_ksplit, persistent, fused_mode;
+    int fused_ok;
+    bool operator==(const PlanKey& o) const
+    {
+        return m == o.m && n == o.n && k == o.k && lda == o.lda && low_bits == o.low_bits && selected == o.selected &&
+               force_variant == o.force_variant && force_ksplit == o.force_ksplit && persistent == o.persistent &&
+               fused_mode == o.fused_mode && fused_ok == o.fused_ok;
+    }
+};
+struct PlanSlot {
+    PlanKey key;
+    Plan plan;
+    bool used = false;
+};
 Plan make_plan(const GemmArgs& g, const Config& cfg)
+{
+    thread_local PlanSlot slots[64];
+    auto low6 = [](const void* p) { return (uint32_t)(reinterpret_cast<uintptr_t>(p) & 63); };
+    const PlanKey key{g.m, g.n, g.k, g.lda,
+                      low6(g.a) | low6(g.b) << 6 | low6(g.a_scale) << 12 | low6(g.b_scale) << 18 | low6(g.c) << 24,
+                      cfg.selected, cfg.force_variant, cfg.force_ksplit, cfg.persistent, cfg.fused_mode, cfg.fused_ok ? 1 : 0};
+    const uint32_t h = ((uint32_t)g.m * 2654435761u) ^ ((uint32_t)g.n * 40503u) ^ ((uint32_t)g.k * 2246822519u) ^
+                       (cfg.fused_ok ? 0x9E3779B9u : 0u);
+    PlanSlot& slot = slots[(h >> 16 ^ h) & 63];
+    if (slot.used && slot.key == key)
+        return slot.plan;
+    slot.plan = compute_plan(g, cfg);
+    slot.key = key;
+    slot.used = true;
+    return slot.plan;
+}
+
+Plan compute_plan(const GemmArgs& g, const Config& cfg)
 {
     const int selected = cfg.selected;
     Plan p{FP8GEMM_KERNEL_SCALAR, 0, 1};
