@@ -28,11 +28,9 @@ namespace fp8gemm {
 
 namespace {
 
-constexpr int QTILE = 128;
-// LDS bytes per k-row of the transposed tile.  33 dwords: the byte stores of a wave (16 k-rows
-// 8 apart, 4 adjacent rows of the source) fall into 8 banks two deep, the dword reads into
-// distinct banks.
-constexpr int QSTRIDE = 132;
+// LDS bytes per k-row of the transposed tile of 128 (64) rows.  33 (17) dwords: the byte stores of a wave (16
+// k-rows 8 apart, 4 adjacent rows of the source) fall into 8 banks two deep, the dword reads into distinct banks.
+constexpr int q_stride(int rows) { return rows + 4; }
 
 __device__ __forceinline__ void load8(const uint16_t* p, float (&v)[8])
 {
@@ -71,12 +69,17 @@ __device__ __forceinline__ float q_value(float x, float scale)
 }
 
 // BLOCK = false: one scale per row and tile (1 x 128).  BLOCK = true: one per tile (128 x 128).
-template <typename TIn, bool BLOCK, bool BF16MATH>
+// QTILE = rows of a workgroup's tile: 128, or 64 for the 1 x 128 quantiser on matrices of a few hundred to a few
+// thousand rows, whose 128-row tiles are too few workgroups to overlap one's loads with another's stores.
+template <typename TIn, bool BLOCK, bool BF16MATH, int QTILE = 128>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __restrict__ scale_out,
                 int rows, int K, int vec_store)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t tile[QTILE * QSTRIDE];
+    static_assert(QTILE == 128 || (QTILE == 64 && !BLOCK), "128 rows, or 64 for the row-wise scales");
+    constexpr int QSTRIDE = q_stride(QTILE);
+    constexpr int PASSES = QTILE / 16;  // rows per thread
+    __shared__ __attribute__((aligned(16))) uint8_t tile[128 * QSTRIDE];
     __shared__ float s_inv[QTILE];
     __shared__ float s_red[4];
 
@@ -86,10 +89,10 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
     const int row0 = blockIdx.x * QTILE;
     const int kb = blockIdx.y;
 
-    float v[8][8];
-    float amax[8];
+    float v[PASSES][8];
+    float amax[PASSES];
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < PASSES; ++p) {
         const int row = row0 + r0 + 16 * p;
         if (row < rows) {
             load8(x + (size_t)row * K + (size_t)kb * 128 + 8 * c, v[p]);
@@ -108,7 +111,7 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
     if (BLOCK) {
         float a = amax[0];
 #pragma unroll
-        for (int p = 1; p < 8; ++p)
+        for (int p = 1; p < PASSES; ++p)
             a = fmaxf(a, amax[p]);
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1)
@@ -118,18 +121,18 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
         __syncthreads();
         a = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
 #pragma unroll
-        for (int p = 0; p < 8; ++p)
+        for (int p = 0; p < PASSES; ++p)
             amax[p] = a;
     } else {
 #pragma unroll
-        for (int p = 0; p < 8; ++p)
+        for (int p = 0; p < PASSES; ++p)
 #pragma unroll
             for (int d = 1; d < 16; d <<= 1)
                 amax[p] = fmaxf(amax[p], __shfl_xor(amax[p], d));
     }
 
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < PASSES; ++p) {
         const int r = r0 + 16 * p;
         const float recip = q_round<BF16MATH>(1.0f / fmaxf(amax[p], q_round<BF16MATH>(1e-12f)));
         const float scale = q_round<BF16MATH>(recip * 448.0f);
@@ -153,17 +156,40 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
     if (!BLOCK && t < QTILE && row0 + t < rows)
         scale_out[(size_t)kb * rows + row0 + t] = s_inv[t];
 
-    // k-row kk of the tile: 128 bytes, one per source row; lane takes 16 of them
-    const int dq = t & 7;
+    // k-row kk of the tile: QTILE bytes, one per source row; lane takes 16 of them
+    constexpr int LPR = QTILE / 16;  // lanes per k-row
+    const int dq = t % LPR;
 #pragma unroll
-    for (int pass = 0; pass < 4; ++pass) {
-        const int kk = (t >> 3) + 32 * pass;
+    for (int pass = 0; pass < 128 * LPR / 256; ++pass) {
+        const int kk = t / LPR + (256 / LPR) * pass;
         const uint32_t* src = reinterpret_cast<const uint32_t*>(tile + kk * QSTRIDE + 16 * dq);
         const uint32_t w[4] = {src[0], src[1], src[2], src[3]};
         const int first = row0 + 16 * dq;
         const size_t o = (size_t)(kb * 128 + kk) * rows + first;
         if (vec_store && first + 16 <= rows) {
             *reinterpret_cast<uint4*>(q + o) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else if (first + 16 <= rows) {
+            // a row count off the 16-byte grid: the piece starts at any byte.  The bytes up to the next dword
+            // boundary one by one, three whole dwords shifted into place, the rest one by one
+            uint8_t* d = q + o;
+            const uint32_t head = (4u - (uint32_t)(reinterpret_cast<uintptr_t>(d) & 3)) & 3;  // 0 ... 3 bytes
+            if (head == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    reinterpret_cast<uint32_t*>(d)[i] = w[i];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 3; ++j)
+                    if ((uint32_t)j < head)
+                        d[j] = (uint8_t)(w[0] >> (8 * j));
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    *reinterpret_cast<uint32_t*>(d + head + 4 * i) = __builtin_amdgcn_alignbyte(w[i + 1], w[i], head);
+#pragma unroll
+                for (int j = 1; j < 4; ++j)  // bytes head + 12 ... 15 are bytes head ... 3 of the last dword
+                    if ((uint32_t)j >= head)
+                        d[12 + j] = (uint8_t)(w[3] >> (8 * j));
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < 16; ++j)
@@ -173,15 +199,21 @@ quantize_kernel(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __res
     }
 }
 
+// 128-row tiles of the 1 x 128 quantiser between these counts run as 64-row tiles
+constexpr long HALF_TILE_LO = 1, HALF_TILE_HI = 2500;
+
 template <typename TIn, bool BF16MATH>
 void launch_quantize_typed(const TIn* x, uint8_t* q, float* scale_out, int rows, int k, bool block128,
                            hipStream_t s)
 {
-    const dim3 grid((rows + QTILE - 1) / QTILE, k / 128);
+    const dim3 grid((rows + 127) / 128, k / 128);
     const int vec_store = (rows % 16 == 0) && (reinterpret_cast<uintptr_t>(q) % 16 == 0);
     if (block128)
         hipLaunchKernelGGL((quantize_kernel<TIn, true, BF16MATH>), grid, dim3(256), 0, s, x, q, scale_out, rows,
                            k, vec_store);
+    else if (HALF_TILE_LO <= (long)grid.x * grid.y && (long)grid.x * grid.y <= HALF_TILE_HI)
+        hipLaunchKernelGGL((quantize_kernel<TIn, false, BF16MATH, 64>), dim3((rows + 63) / 64, k / 128), dim3(256), 0, s, x,
+                           q, scale_out, rows, k, vec_store);
     else
         hipLaunchKernelGGL((quantize_kernel<TIn, false, BF16MATH>), grid, dim3(256), 0, s, x, q, scale_out, rows,
                            k, vec_store);

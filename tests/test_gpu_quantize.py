@@ -52,8 +52,10 @@ def _check(pkg, x, which, dtype):
     assert bad.size == 0, (which, x.shape, bad[:4], q[tuple(bad[0])], rq[tuple(bad[0])])
 
 
+# (row counts off the 16-byte grid leave through dword stores shifted into place: odd, 2 mod 4, 0 mod 4;
+# 20001 x 2048 is past the tile count up to which the 1 x 128 quantiser works in 64-row tiles)
 SHAPES_A = [(32, 2048), (1024, 2048), (2048, 7168), (16, 128), (1, 128), (130, 256), (77, 384),
-            (200, 128)]
+            (200, 128), (1001, 512), (259, 256), (3, 256), (20001, 2048), (16384, 2560)]
 SHAPES_B = [(512, 2048), (576, 7168), (7168, 2048), (128, 128), (64, 128), (1, 256), (130, 256),
             (300, 384)]
 
