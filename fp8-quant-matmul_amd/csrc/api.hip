@@ -349,11 +349,12 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
         if (wide_ok && (by_name ? cfg.force_variant != 0 : cfg.force_variant < 0)) {
             // without the in-kernel reduction (no zeroed mailbox, or workgroup placement not confirmed) only
             // the unsplit form exists.  By name, tile_variant 2 pins the 256-column strips.
-            // Left to the cost model, 256-column strips have to be 7 % ahead in launches of a single round: they
-            // halve the workgroups of a split and win where that saves a round (144 strips x 3 splits are 54
-            // workgroups on an XCD's 32 CUs, 72 x 3 are 27: 18432 x 7168 from HBM 28.6 against 34.6 us), and lose
-            // 15 - 40 % on cfg5-sized problems.  Launches of several rounds stream, and there the wider strips are
-            // ahead throughout (a projection onto a vocabulary with 8 rows, 131072 x 4096: 93.3 against 101.7 us).
+            // Left to the cost model, 256-column strips have to be 7 % ahead where K is split: they halve the
+            // workgroups of a split and win where that saves a round (144 strips x 3 splits are 54 workgroups on
+            // an XCD's 32 CUs, 72 x 3 are 27: 18432 x 7168 from HBM 28.6 against 34.6 us), and lose 15 - 40 % on
+            // cfg5-sized problems.  Unsplit launches stream, and there the wider strips are ahead throughout (a
+            // projection onto a vocabulary with 8 rows, 131072 x 4096: 93.3 against 101.7 us; 16 x 49152 x 4096 in
+            // one round of 192 workgroups 39.0 us, against 48.4 us in 384 strips of 128 columns).
             const int hi = cfg.fused_ok ? (nkb < MAX_KSPLIT ? nkb : MAX_KSPLIT) : 1;
             for (int halves = 1; halves <= 2; ++halves) {
                 if (by_name ? halves != (cfg.force_variant == 2 ? 2 : 1) : cfg.force_variant >= 0 && halves == 2)
@@ -361,9 +362,8 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
                 for (int ks = 1; ks <= hi; ++ks) {
                     if (!valid_split(ks) || (forced_ks && ks != forced_ks) || !decode_strip_can_split(g, ks, halves))
                         continue;
-                    const long per_xcd = (long)(((g.n + 255) / 256 + 7) / 8) * ks;  // workgroups of 256-column strips
                     const double cst =
-                        decode_strip_cost(g, ks, halves) * (halves == 2 && !by_name && (per_xcd <= 32 || ks > 1) ? 1.07 : 1.0);
+                        decode_strip_cost(g, ks, halves) * (halves == 2 && !by_name && ks > 1 ? 1.07 : 1.0);
                     if (cst < wide_us) {
                         wide_us = cst;
                         wide.ksplit = ks;

@@ -804,6 +804,20 @@ double decode_strip_cost(const GemmArgs& g, int ksplit, int halves)
     const int strips = (g.n + DS_BN * halves - 1) / (DS_BN * halves);
     const int nkb = g.k / KBLOCK;
     const int kbs = (nkb + ksplit - 1) / ksplit;
+    // An unsplit launch of more strips than the device holds workgroups: 256 workgroups at a time take the strips
+    // in turn (the streaming form, which makes them 256 columns wide once there are 256 such strips; with rows off
+    // the 16-byte grid the plain kernel's workgroups as CUs free up), a full turn at what HBM delivers (1.33 us
+    // per K block of 256-column strips, 0.756 us of 128-column ones), the last, partial turn like a launch of
+    // that many workgroups.  (16 x 65792 / 81920 / 98304 x 2048: 32.8 / 36.1 / 39.4 us estimated, 31.2 / 38.7 /
+    // 41.2 us measured; 8 x 131072 x 4096: 88.6, 92.9 us; 8 x 163840 x 2048 in 256-column strips 60.6, 64.9 us, in
+    // 128-column strips 64.0, 72.6 us.)
+    if (ksplit == 1 && strips > STREAM_WORKGROUPS) {
+        const long wide_units = (g.n + 2 * DS_BN - 1) / (2 * DS_BN);
+        const bool wide = halves == 2 || (leading_dim(g) % 16 == 0 && wide_units >= STREAM_WORKGROUPS);
+        const long units = wide ? wide_units : strips;
+        const long turns = units / STREAM_WORKGROUPS, tail = units % STREAM_WORKGROUPS;
+        return 3.5 + kbs * (turns * (wide ? 1.33 : 0.756) + (tail ? 0.50 + (wide ? 0.0032 : 0.001) * tail : 0.0));
+    }
     const long wgs = (long)strips * ksplit;
     // the splits of a strip share an XCD (32 CUs, one workgroup each), strips are dealt out over the eight XCDs:
     // 36 strips x 7 splits are 252 workgroups, but 35 on each of four XCDs, which is two rounds there (measured:
@@ -813,7 +827,12 @@ double decode_strip_cost(const GemmArgs& g, int ksplit, int halves)
     // (a stage of a 256-column strip is twice the bytes for 1.92 times the time in a launch of one round, which
     // lives on latencies, and for 1.8 times in longer unsplit ones, which stream: 256 contiguous bytes come 10 %
     // faster)
-    const double per_block = (0.50 + 0.001 * active) * (halves == 2 ? (rounds > 1 && ksplit == 1 ? 1.8 : 1.92) : 1.0);
+    double per_block = (0.50 + 0.001 * active) * (halves == 2 ? (rounds > 1 && ksplit == 1 ? 1.8 : 1.92) : 1.0);
+    // (one round of unsplit 256-column strips streams its whole K range and is bound by what HBM delivers to all
+    // of them: 0.81 / 0.99 / 1.06 / 1.22 us per block with 129 / 160 / 192 / 224 workgroups -- 33024 ... 57344
+    // columns, K = 2048 and 8192 -- which is 5.1 ... 5.9 TB/s)
+    if (halves == 2 && ksplit == 1 && rounds == 1)
+        per_block = 0.50 + 0.0032 * active;
     const double life = 1.0 + kbs * per_block + (ksplit > 1 ? 0.39 * ksplit : 0.0);
     return 2.5 + (double)rounds * life;
 }
@@ -867,10 +886,12 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, int halves, float
                            leading_dim(g), g.n, g.k, strips, ksplit, kb_per_split);
         return hipGetLastError();
     };
-    // more 128-column strips than resident workgroups, no K split: one copy stream per workgroup (the streaming
-    // form chooses its strip width itself)
+    // more strips than resident workgroups, no K split: one copy stream per workgroup (the streaming form chooses
+    // its strip width itself).  Strips of the width asked for: 57344 columns are 448 strips of 128 -- two turns of
+    // the streaming workgroups, the second three quarters full, 96.9 us for 16 x 57344 x 8192 -- but 224 strips of
+    // 256, one round of plain workgroups, 80.8 us.
     const int strips128 = (g.n + DS_BN - 1) / DS_BN;
-    if (ksplit == 1 && strips128 > STREAM_WORKGROUPS && leading_dim(g) % 16 == 0) {
+    if (ksplit == 1 && strips > STREAM_WORKGROUPS && leading_dim(g) % 16 == 0) {
         const bool staged = reinterpret_cast<uintptr_t>(g.c) % 16 == 0;
         const int wide_units = (g.n + 2 * DS_BN - 1) / (2 * DS_BN);
         const bool wide = wide_units >= STREAM_WORKGROUPS;  // 256-column strips while every CU gets one

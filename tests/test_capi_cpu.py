@@ -248,6 +248,11 @@ def test_dispatcher_plans(pkg):
     # 72 x 3: 27) and in unsplit launches of several rounds (a projection onto a vocabulary)
     assert pkg.plan(32, 18432, 7168) == "decode256_k3"
     assert pkg.plan(8, 131072, 4096) == "decode256_k1"
+    # 129 ... 256 strips of 256 columns unsplit: one round that streams (384 strips of 128 would take two turns)
+    assert pkg.plan(16, 49152, 4096) == "decode256_k1"
+    assert pkg.plan(16, 57344, 8192) == "decode256_k1"
+    assert pkg.plan(8, 81920, 2048) == "decode256_k1"      # rows off the grid, several rounds: the wider strips
+    assert pkg.plan(16, 28672, 4096) == "decode128_k1"     # 224 strips of 128: one round
     assert pkg.plan(32, 7168, 7168) == "decode128_k4"
     pkg.select(pkg.KERNEL_SKINNY)
     pkg.force_config(-1, 3)
