@@ -762,6 +762,7 @@ struct StreamShape {
     static constexpr int MT = MT_, NS = NS_, NB = NB_;
 };
 constexpr int STREAM_WORKGROUPS = 256;
+constexpr int SLAB_FORM_MIN_KBLOCKS = 28;  // K blocks per workgroup from which up to 32 rows on the grid take the slab-spreading instances too
 
 // Two workgroups per CU with a three-stage ring instead of one with six: one streams while the other starts up.
 // Measured on grouped launches: 64 groups x 56 strips, 16 K blocks each: 221 against 236 us; with 768-1152
@@ -940,7 +941,12 @@ hipError_t launch_decode_strips(const GemmArgs& g, int ksplit, int halves, float
         return leading_dim(g) % 16 != 0 ? by_tiles(std::true_type{}) : by_tiles(std::false_type{});
     }
     const int tiles = (g.m + 15) / 16;
-    if (leading_dim(g) % 16 != 0) {
+    // The instances that spread A's packed slabs take rows on the grid as well, and a workgroup with a long K
+    // range runs 3 - 8 % faster in them (28672 x 8192 unsplit, 15 / 16 / 31 / 32 rows: 43.2 / 45.8 / 45.1 / 47.1 us;
+    // 16384 x 7168 in two splits, 47 / 48 rows: 26.3 / 27.8 us), a short one 3 - 10 % slower (24576 x 2048 unsplit,
+    // 31 / 32 rows: 14.4 / 13.9 us; 7168 x 2048 in four splits: 8.0 / 7.3 us).  With three or four row tiles the
+    // two measure level (their slab form has a ring of four stages, not six).
+    if (leading_dim(g) % 16 != 0 || (kb_per_split >= SLAB_FORM_MIN_KBLOCKS && tiles <= 2)) {
         constexpr int L2 = DecodeShape<2, 6, true>::LDS, L4 = DecodeShape<4, RAGGED4_NS, true>::LDS;
         switch (tiles) {
         case 1: return go(decode_strip_kernel<2, 6, true, 1, 1>, L2);

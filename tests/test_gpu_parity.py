@@ -330,6 +330,25 @@ def test_decode_rows_off_the_grid_run_without_a_padded_copy(pkg):
 # 256-column strips (tile_variant 2 of the decode family): two 128-column halves per stage, their own b_scale
 # each; strips whose last one ends in its first half / in its second; every row-tile count, rows on and off the
 # 16-byte grid; split and unsplit; results bit-identical to the 128-column strips with the same K split
+# rows on the 16-byte grid with 28 or more K blocks per workgroup run in the instances that spread A's packed slabs
+DECODE_LONG_K_CASES = [(16, 2048, 4096, 1), (32, 1536, 7168, 2), (48, 640, 3584, 1), (64, 1024, 7168, 2), (32, 256, 8192, 2)]
+
+
+@pytest.mark.parametrize("m,n,k,ksplit", DECODE_LONG_K_CASES)
+def test_decode_rows_on_the_grid_with_a_long_k_range_per_workgroup(pkg, m, n, k, ksplit):
+    a, b, sa, sb = oracle.make_inputs(m, n, k, 1370 + m + n + k + ksplit, 0.5, 30.0)
+    ref = oracle.ref_gemm(a, b, sa, sb, m, n, k)
+    got, name = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=1, ksplit=ksplit)
+    assert name == f"decode128_k{ksplit}", name
+    _assert_close(got, ref, name)
+    _assert_every_element(got, a, b, sa, sb, m, n, k, name)
+    # the same K split with fewer K blocks per workgroup is not available; the 256-column strips (plain instances
+    # at any K range) give the same bits
+    wide, wname = _run(pkg, a, b, sa, sb, m, n, k, kernel=pkg.KERNEL_SKINNY, variant=2, ksplit=ksplit)
+    assert wname == f"decode256_k{ksplit}", wname
+    assert np.array_equal(got, wide), "slab-spreading instance and plain 256-column instance differ"
+
+
 DECODE_WIDE_STRIP_CASES = [(32, 7168, 2048, 4), (16, 7168, 2048, 1), (32, 576, 1024, 3), (32, 1200, 2048, 16),
                            (7, 4608, 7168, 6), (40, 2064, 7168, 8), (63, 256, 128, 1), (1, 18432, 1024, 2),
                            (24, 16384, 1024, 4), (48, 7168, 2048, 2), (64, 112, 512, 2), (33, 18432, 384, 3)]
