@@ -468,6 +468,12 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
             if (g.m <= 64 && fk <= 0 && selected == FP8GEMM_KERNEL_AUTO && ks > 1 &&
                 kbs < (tile_plan_fused(g, v, ks, cfg) ? 3 : 8))
                 continue;
+            // 128x128 tiles that add their splits inside the kernel hand over 64 KB per split: with fewer than 8 K
+            // blocks per workgroup that costs more than the split saves (27 shapes with K = 1536, 96 ... 128 tiles,
+            // two splits of 6 blocks against unsplit: 10 - 28 % slower with B cached, -2 ... +15 % from HBM)
+            if (v == TILE_128x128 && ks > 1 && kbs < 8 && fk <= 0 && selected == FP8GEMM_KERNEL_AUTO &&
+                tile_plan_fused(g, v, ks, cfg))
+                continue;
             const double cst = tile_cost(g, v, ks, tile_plan_fused(g, v, ks, cfg));
             if (cst < best) {
                 best = cst;

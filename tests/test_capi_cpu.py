@@ -228,6 +228,8 @@ def test_dispatcher_plans(pkg):
     # more than one round
     assert pkg.plan(2144, 608, 3072) == "tile128x128_k2f"
     assert pkg.plan(2048, 576, 3072) == "tile128x128_k3f"  # 80 tiles x 3: one round
+    # 128x128 tiles do not split into ranges of fewer than 8 K blocks (64 KB per split to hand over)
+    assert pkg.plan(1024, 2048, 1536) == "tile128x128_k1"
     # 129 ... 256 rows over 32 MB of B or more: one row of 256x128 tiles streams B once
     assert pkg.plan(208, 18816, 3072) == "tile256x128_k1"
     assert pkg.plan(400, 11648, 7168) == "tile128x192_k1"  # more rows: the cost model's tile
