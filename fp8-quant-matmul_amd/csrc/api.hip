@@ -434,7 +434,8 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
                 decide_fused(g, p, cfg);
                 return p;
             }
-    double best = 1e300;
+    double best = 1e300, best_256x128 = 1e300;
+    int ks_256x128 = 1;
     for (int v = 0; v < TILE_VARIANT_COUNT; ++v) {
         if (fv >= 0 && v != fv)
             continue;
@@ -481,6 +482,10 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
                 p.variant = v;
                 p.ksplit = ks;
             }
+            if (v == TILE_256x128 && cst < best_256x128) {
+                best_256x128 = cst;
+                ks_256x128 = ks;
+            }
         }
     }
     if (decode_us >= 0.0 && decode_us <= 0.95 * best)  // measured: at equal estimates the decode kernel is ahead
@@ -489,7 +494,17 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
         p.family = -1;
         return p;
     }
-    // 129 ... 256 rows over a B of 32 MB or more: one row of 256x128 tiles streams B once where the 128x192 tile
+    // 129 ... 256 rows over a B of 32 MB or more: 128-row tiles read B twice, one row of 256x128 tiles once.  Where
+    // the model takes 128x128 tiles with a 256x128 plan within 12 % of them, that plan -- mostly two splits with
+    // the reduction kernel -- measures 4 - 16 % ahead with B cached and 3 - 29 % with B from HBM (30 random shapes,
+    // all ahead in both; 192 x 14720 x 7168, 160 x 15104 x 8192).
+    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && p.variant == TILE_128x128 && g.m > 128 && g.m <= 256 &&
+        (long long)g.n * g.k >= 32000000ll && best_256x128 <= 1.12 * best) {
+        p.variant = TILE_256x128;
+        p.ksplit = ks_256x128;
+        p.family = p.ksplit > 1 ? FP8GEMM_KERNEL_SPLITK : FP8GEMM_KERNEL_LARGE;
+    }
+    // The same rows where the model takes the 128x192 tile: one row of 256x128 tiles streams B once where the 128x192 tile
     // the fit to cached operands prefers reads it twice.  With B from HBM -- which is what such a B is in a
     // model -- the taller tile is 2 - 13 % ahead on 22 random shapes (208 x 18816 x 3072: +12.8 %), with B in the
     // Infinity Cache -5 ... +4 %; with more rows (two to four tile rows against four to eight) the two are level.

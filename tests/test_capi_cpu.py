@@ -232,6 +232,8 @@ def test_dispatcher_plans(pkg):
     assert pkg.plan(1024, 2048, 1536) == "tile128x128_k1"
     # 129 ... 256 rows over 32 MB of B or more: one row of 256x128 tiles streams B once
     assert pkg.plan(208, 18816, 3072) == "tile256x128_k1"
+    assert pkg.plan(192, 14720, 7168) == "tile256x128_k2"   # ... where the model would take 128x128 tiles as well
+    assert pkg.plan(256, 7168, 7168) == "tile128x128_k2f"   # no 256x128 plan within reach: stays
     assert pkg.plan(400, 11648, 7168) == "tile128x192_k1"  # more rows: the cost model's tile
     # decode shapes (M <= 32): 128-column strips with the K range split so that one round of workgroups
     # (at most 256) streams B, the splits added inside the kernel
