@@ -494,12 +494,14 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
         p.family = -1;
         return p;
     }
-    // 129 ... 256 rows over a B of 32 MB or more: 128-row tiles read B twice, one row of 256x128 tiles once.  Where
-    // the model takes 128x128 tiles with a 256x128 plan within 12 % of them, that plan -- mostly two splits with
-    // the reduction kernel -- measures 4 - 16 % ahead with B cached and 3 - 29 % with B from HBM (30 random shapes,
-    // all ahead in both; 192 x 14720 x 7168, 160 x 15104 x 8192).
-    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && p.variant == TILE_128x128 && g.m > 128 && g.m <= 256 &&
-        (long long)g.n * g.k >= 32000000ll && best_256x128 <= 1.12 * best) {
+    // 129 ... 512 rows over a B of 16 MB or more with a long K: 128-row tiles read B twice as often as 256-row
+    // tiles.  Where the model takes 128x128 tiles with a 256x128 plan within 12 % of them, that plan -- mostly two
+    // to four splits with the reduction kernel -- measures ahead with B cached and with B from HBM: 45 random
+    // shapes of up to 256 rows over 32 MB or more all faster, by 12 and 17 % on average; 56 more of up to 512 rows
+    // or 18 ... 32 MB with K >= 4096: +8.3 and +6.4 % on average, worst -3.8 % (K = 3072, where an unsplit 128x128
+    // plan would give way to three splits, loses 4 - 10 % and is left out).
+    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && p.variant == TILE_128x128 && g.m > 128 && g.m <= 512 &&
+        g.k >= 4096 && (long long)g.n * g.k >= 16000000ll && best_256x128 <= 1.12 * best) {
         p.variant = TILE_256x128;
         p.ksplit = ks_256x128;
         p.family = p.ksplit > 1 ? FP8GEMM_KERNEL_SPLITK : FP8GEMM_KERNEL_LARGE;
