@@ -494,13 +494,14 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
         p.family = -1;
         return p;
     }
-    // 129 ... 512 rows over a B of 16 MB or more with a long K: 128-row tiles read B twice as often as 256-row
+    // 129 ... 1536 rows over a B of 16 MB or more with a long K: 128-row tiles read B twice as often as 256-row
     // tiles.  Where the model takes 128x128 tiles with a 256x128 plan within 12 % of them, that plan -- mostly two
     // to four splits with the reduction kernel -- measures ahead with B cached and with B from HBM: 45 random
     // shapes of up to 256 rows over 32 MB or more all faster, by 12 and 17 % on average; 56 more of up to 512 rows
     // or 18 ... 32 MB with K >= 4096: +8.3 and +6.4 % on average, worst -3.8 % (K = 3072, where an unsplit 128x128
-    // plan would give way to three splits, loses 4 - 10 % and is left out).
-    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && p.variant == TILE_128x128 && g.m > 128 && g.m <= 512 &&
+    // plan would give way to three splits, loses 4 - 10 % and is left out); 49 of 528 ... 1536 rows: +7.4 and +6.1 %, worst
+    // -3.0 %.
+    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && p.variant == TILE_128x128 && g.m > 128 && g.m <= 1536 &&
         g.k >= 4096 && (long long)g.n * g.k >= 16000000ll && best_256x128 <= 1.12 * best) {
         p.variant = TILE_256x128;
         p.ksplit = ks_256x128;
