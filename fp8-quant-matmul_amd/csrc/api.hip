@@ -500,8 +500,8 @@ Plan compute_plan(const GemmArgs& g, const Config& cfg)
     // shapes of up to 256 rows over 32 MB or more all faster, by 12 and 17 % on average; 56 more of up to 512 rows
     // or 18 ... 32 MB with K >= 4096: +8.3 and +6.4 % on average, worst -3.8 % (K = 3072, where an unsplit 128x128
     // plan would give way to three splits, loses 4 - 10 % and is left out); 49 of 528 ... 1536 rows: +7.4 and +6.1 %, worst
-    // -3.0 %.
-    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && p.variant == TILE_128x128 && g.m > 128 && g.m <= 1536 &&
+    // -3.0 %.  The same where the model takes a 128x192 plan with splits: 56 shapes, +3.6 and +7.4 %, worst -4.6 %.
+    if (selected == FP8GEMM_KERNEL_AUTO && fv < 0 && fk <= 0 && (p.variant == TILE_128x128 || p.variant == TILE_128x192) && g.m > 128 && g.m <= 1536 &&
         g.k >= 4096 && (long long)g.n * g.k >= 16000000ll && best_256x128 <= 1.12 * best) {
         p.variant = TILE_256x128;
         p.ksplit = ks_256x128;
