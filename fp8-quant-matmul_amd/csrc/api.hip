@@ -188,7 +188,11 @@ double tile_cost(const GemmArgs& g, int variant, int ksplit, bool fused = false)
     const bool light = variant == TILE_64x64 && !streams_b && tiles <= 64;
     const double per_kb = (1.19 * area + 0.267) * (variant == TILE_256x256 ? 1.03 : 1.0) * (streams_b ? 1.25 : 1.0) *
                           (light ? 0.8 : 1.0);
-    const double per_item = 0.95 + 4.38 * area + kbs * per_kb;
+    // (unsplit 128x192 tiles in more than one round of workgroups: the fit has them 8 % too fast against the 256-row
+    // tiles -- 36 random shapes of 512 ... 8192 rows where that margin decides, before / after: the 256x256 or
+    // 256x128 plan +5.6 % with B cached, +10.3 % with B from HBM on average, worst -2.3 %)
+    const double in_rounds = variant == TILE_128x192 && ksplit == 1 && tiles > NUM_CU ? 1.08 : 1.0;
+    const double per_item = 0.95 + 4.38 * area + kbs * per_kb * in_rounds;
     // (two 64x64 workgroups share a CU, but a single row of tiles with B from HBM is fastest with at most one
     // workgroup per CU: M = 48, 64 on 12 shapes, the split that keeps tiles x splits within 256 is the best
     // measured or within 2 % of it)
